@@ -147,6 +147,9 @@ class HybridArch:
     # the stream that enters the next layer is a learned average of all earlier layers' results
     arrangement: str = "gated_parallel"
     depth_average: bool = False
+    # copies of the residual stream a layer reads and writes through learned weights (1: one plain stream);
+    # the ``hyper_pre_norm`` arrangement uses them
+    streams: int = 1
 
     @property
     def num_layers(self) -> int:
@@ -237,8 +240,65 @@ def _pozalorn_from_config(cfg: dict, name: str) -> HybridArch:
                       arrangement="post_norm", depth_average=True)
 
 
+def _livitar_mixer(kind: str, m: dict) -> tuple:
+    """(key of ``vgate.models.mixers.MIXERS``, its spec) of a Livitar layer type. What the design fixes
+    (which norm, which gate, how positions enter) is written out here as options of the general mixers."""
+    if kind == "retention":   # constant decay per head, half-split rotary positions on q / k, keys scaled by dim^-1/2
+        dec = [float(d) for d in m["decay"]]
+        if len(dec) != int(m["heads"]):
+            raise ValueError("retention: one decay per head")
+        rot = m.get("rot") or {}
+        return "linear_attention", {"heads": int(m["heads"]), "dim": int(m["dim"]), "vdim": int(m["vdim"]),
+                                    "decay": {"kind": "head", "values": dec}, "q_scale": 1.0, "k_scale": float(m["dim"]) ** -0.5,
+                                    "rot": {"dims": int(rot.get("dims", 0)), "base": float(rot.get("base", 10000.0)), "layout": "half"},
+                                    "in_act": "none", "out_norm": "head", "norm_weight": False, "gate_act": "silu"}
+    if kind in ("attention", "attention_2"):   # full causal softmax attention without rotation, sigmoid output gate
+        spec = {"heads": int(m["heads"]), "kv_heads": int(m["kv_heads"]), "dim": int(m["dim"]), "vdim": int(m["vdim"]),
+                "scale": float(m["scale"]), "rot": {"dims": 0}, "window": None, "gate": "sigmoid"}
+        if kind == "attention":   # per-head temperature; penalty r1 ln(1 + r2 distance)
+            spec.update(qk_norm="none", head_temp=True, dist_bias={"kind": "log"})
+        else:                     # unit-RMS q / k; query temperature growing with the position; learned bias per distance bucket
+            qt = m["q_temp"]
+            spec.update(qk_norm="head", qk_norm_weight=False, q_temp={"coef": float(qt["coef"]), "every": int(qt["every"])},
+                        dist_bias={"kind": "table", "far": float(m["bias_max"])})
+        return "window_attention", spec
+    raise ValueError(f"Livitar has no layer type {kind!r}")
+
+
+def _livitar_mlp(mlp: dict | None) -> dict | None:
+    if not mlp:
+        return None
+    if mlp.get("kind") != "moe":
+        raise ValueError(f"Livitar feed-forward kind {mlp.get('kind')!r}")
+    r = mlp["router"]
+    out = {"kind": "moe", "expert": {"ff": int(mlp["expert"]["ff"]), "act": "silu"},
+           "router": {"experts": int(r["experts"]), "top": int(r["top"]), "scale": float(r.get("scale", 1.0)),
+                      "score": "softmax", "correction": False}}
+    if mlp.get("shared"):
+        out["shared"] = {"ff": int(mlp["shared"]["ff"])}
+    return out
+
+
+def _livitar_from_config(cfg: dict, name: str) -> HybridArch:
+    """config.json of the Livitar design: pre-norm layers with a tanh norm (no statistics) over several
+    copies of the residual stream that every sublayer reads, mixes and writes through learned weights;
+    mixers: retention, and two kinds of full causal attention whose positions enter as a bias on the scores."""
+    layers = []
+    for L in cfg["layers"]:
+        kind, spec = _livitar_mixer(L["type"], L["mixer"])
+        layers.append(LayerSpec(kind=kind, mixer=spec, mlp=_livitar_mlp(L.get("mlp"))))
+    eos = cfg.get("eos_token_id", 2)
+    streams = int(cfg.get("streams", 1))
+    if streams < 1:
+        raise ValueError("streams >= 1")
+    return HybridArch(name=name, family="livitar", hidden_size=int(cfg["width"]), vocab_size=int(cfg["vocab"]),
+                      layers=tuple(layers), rms_eps=float(cfg["norm"]["eps"]), bos_token_id=int(cfg.get("bos_token_id", 1)),
+                      eos_token_ids=tuple(eos) if isinstance(eos, list) else (int(eos),),
+                      arrangement="hyper_pre_norm", streams=streams)
+
+
 # config.json "architecture" -> parser of a layered hybrid design
-HYBRID_ARCHITECTURES = {"Zadirax": _zadirax_from_config, "Pozalorn": _pozalorn_from_config}
+HYBRID_ARCHITECTURES = {"Zadirax": _zadirax_from_config, "Pozalorn": _pozalorn_from_config, "Livitar": _livitar_from_config}
 
 
 def _zadirax_preset(name: str, width: int, vocab: int, pairs: int, heads: int, dim: int, ff: int, experts: int,
@@ -277,6 +337,26 @@ def _pozalorn_preset(name: str, width: int, vocab: int, groups: int, heads: int,
     return _pozalorn_from_config(cfg, name)
 
 
+def _livitar_preset(name: str, width: int, vocab: int, groups: int, heads: int, kv_heads: int, dim: int, experts: int,
+                    top: int, expert_ff: int, shared_ff: int, streams: int = 2, ret_heads: int | None = None,
+                    buckets_far: int = 1024) -> HybridArch:
+    """Random-init Livitar models (benchmarks, tests): ``groups`` x [retention, attention, attention_2], each
+    with a mixture-of-experts feed-forward and a shared expert."""
+    rh = ret_heads or heads
+    mlp = {"kind": "moe", "expert": {"ff": expert_ff}, "router": {"experts": experts, "top": top, "scale": 1.5},
+           "shared": {"ff": shared_ff}}
+    ret = {"type": "retention", "mlp": mlp,
+           "mixer": {"heads": rh, "dim": dim, "vdim": dim, "rot": {"base": 10000.0, "dims": dim},
+                     "decay": [1.0 - 2.0 ** (-5.0 - 6.0 * i / max(rh - 1, 1)) for i in range(rh)]}}
+    a1 = {"type": "attention", "mlp": mlp,
+          "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5}}
+    a2 = {"type": "attention_2", "mlp": mlp,
+          "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                    "bias_max": buckets_far, "q_temp": {"coef": 0.1, "every": 128}}}
+    cfg = {"width": width, "vocab": vocab, "streams": streams, "norm": {"eps": 1e-6}, "layers": [ret, a1, a2] * groups}
+    return _livitar_from_config(cfg, name)
+
+
 HYBRID_PRESETS = {
     # tests / CPU smoke: odd sizes on purpose (nothing a multiple of the MFMA tile)
     "zadirax-tiny": lambda: _zadirax_preset("zadirax-tiny", 96, 300, 2, 3, 24, 136, 5, 2, 40, 56, 40, 8, share=True),
@@ -289,6 +369,11 @@ HYBRID_PRESETS = {
     # slices at the layer sizes of real models beside a transformer of equal width (benchmarks/design_compare.py)
     "pozalorn-bench-1024": lambda: _pozalorn_preset("pozalorn-bench-1024", 1024, 32000, 1, 8, 2, 128, 4096, 1024, 64),
     "pozalorn-bench-1536": lambda: _pozalorn_preset("pozalorn-bench-1536", 1536, 32000, 1, 12, 2, 128, 8960, 1024, 64),
+    # tests / CPU smoke: odd sizes on purpose
+    "livitar-tiny": lambda: _livitar_preset("livitar-tiny", 88, 300, 1, 4, 2, 24, 5, 2, 40, 56, streams=3, ret_heads=3, buckets_far=50),
+    # slices at the layer sizes of real models beside a transformer of equal width (benchmarks/design_compare.py)
+    "livitar-bench-1024": lambda: _livitar_preset("livitar-bench-1024", 1024, 32000, 1, 8, 2, 128, 8, 2, 2048, 2048),
+    "livitar-bench-1536": lambda: _livitar_preset("livitar-bench-1536", 1536, 32000, 1, 12, 2, 128, 16, 4, 2240, 2240),
     # layer sizes of a ~1.5B model (the width, head size, feed-forward and vocabulary of qwen2.5-1.5b)
     "zadirax-1.5b": lambda: _zadirax_preset("zadirax-1.5b", 1536, 151936, 14, 12, 128, 8960, 32, 4, 2240, 512, 768, 64),
 }

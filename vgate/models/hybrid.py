@@ -12,6 +12,11 @@ Layer arrangements (``ARRANGEMENTS``, chosen by ``HybridArch.arrangement``):
   post_norm       x += rmsnorm(mixer(x)) * w1;  x += rmsnorm(ff(x)) * w2
                   (the sublayers read the stream itself, rounded to the activation dtype; their
                   outputs are normed in fp32 before they are added)
+  hyper_pre_norm  ``HybridArch.streams`` fp32 copies x_1 .. x_S of the stream (all equal to the embedding
+                  output at the start); per sublayer q with a tanh norm (no statistics):
+                  u = sum_s in_q[s] x_s;  y = sublayer(tanh(alpha u) * w + b);
+                  x_t <- sum_s mix_q[s, t] x_s + out_q[t] y   (all copies at once); the model's result
+                  is the sum of the copies
 With ``HybridArch.depth_average`` the stream a layer hands on is a learned combination of the
 embedding output X_0 and every layer result X_1 .. X_(i+1): sum_j c_i[j] X_j (tensor ``l<i>.dwa``).
 A layer may run with another layer's weights (``weights_of``) while keeping its own cache or state.
@@ -150,7 +155,96 @@ class PostNormLayer:
             seq.post_norm_add(st.result, yf, self.norm2, self.eps, st.result, **st.hand_on(True))
 
 
-ARRANGEMENTS = {"gated_parallel": GatedParallelLayer, "post_norm": PostNormLayer}
+class _TanhNorm:
+    """tanh(alpha x) * w + b: the tensors ``<name>`` [W], ``<name>.b`` [W], ``<name>.alpha`` []."""
+
+    def __init__(self, t: dict, name: str, device):
+        self.alpha = _f32(t[name + ".alpha"].reshape(1), device)
+        self.w, self.b = _f32(t[name], device), _f32(t[name + ".b"], device)
+
+    @staticmethod
+    def shapes(name: str, width: int) -> dict:
+        return {name: (width,), name + ".b": (width,), name + ".alpha": ()}
+
+
+class HyperPreNormLayer:
+    """``hyper_pre_norm`` arrangement: every sublayer reads a learned combination of the stream's copies
+    through a tanh norm and writes back to all of them (tensors ``hc<q>.in`` [S], ``hc<q>.out`` [S],
+    ``hc<q>.mix`` [S from, S to]). A sublayer's write and the next sublayer's read (also the next layer's,
+    or the final sum over the copies) are one kernel."""
+
+    def __init__(self, spec, width: int, eps: float, t: dict, device, f32: bool):
+        mix = {k[4:]: v for k, v in t.items() if k.startswith("mix.")}
+        self.eps = eps
+        if spec.kind == "parallel":
+            raise ValueError("the hyper_pre_norm arrangement takes single mixers")
+        self.mixer = MIXERS[spec.kind](spec.mixer, width, eps, mix, device, f32)
+        self.norm1 = _TanhNorm(t, "norm1", device)
+        self.hc = [tuple(_f32(t[f"hc1.{n}"], device) for n in ("in", "out", "mix"))]
+        self.ff = self.norm2 = None
+        if spec.mlp:
+            mlp = {k[4:]: v for k, v in t.items() if k.startswith("mlp.")}
+            self.ff = FEED_FORWARDS[spec.mlp["kind"]](spec.mlp, width, mlp, device, f32)
+            self.norm2 = _TanhNorm(t, "norm2", device)
+            self.hc.append(tuple(_f32(t[f"hc2.{n}"], device) for n in ("in", "out", "mix")))
+        S = self.hc[0][0].numel()
+        if S > seq.MAX_STREAMS or any(c[2].shape != (S, S) or c[1].numel() != S for c in self.hc):
+            raise ValueError(f"hyper_pre_norm: 1 .. {seq.MAX_STREAMS} copies, mix [copies, copies]")
+        self.proj, self.col = _fuse_inputs(self.mixer, [], width, device, f32)
+
+    @staticmethod
+    def shapes(spec, width: int, streams: int = 1) -> dict:
+        hc = lambda q: {f"hc{q}.in": (streams,), f"hc{q}.out": (streams,), f"hc{q}.mix": (streams, streams)}  # noqa: E731
+        out = dict(_TanhNorm.shapes("norm1", width))
+        out.update({"mix." + k: v for k, v in MIXERS[spec.kind].shapes(spec.mixer, width).items()})
+        out.update(hc(1))
+        if spec.mlp:
+            out.update({"mlp." + k: v for k, v in FEED_FORWARDS[spec.mlp["kind"]].shapes(spec.mlp, width).items()})
+            out.update(_TanhNorm.shapes("norm2", width))
+            out.update(hc(2))
+        return out
+
+    def cols(self, P: torch.Tensor, name: str) -> torch.Tensor:
+        a, n = self.col[name]
+        return P[:, a: a + n]
+
+    def nbytes(self) -> int:
+        return self.proj.nbytes() + self.mixer.nbytes() + (self.ff.nbytes() if self.ff else 0)
+
+    def reader(self) -> tuple:
+        """What the kernel before this layer needs to prepare its first sublayer's input."""
+        return self.hc[0][0], self.norm1
+
+    def run(self, st, sv, cache) -> None:
+        """st.xs [S, T, W]: the copies; st.h: the first sublayer's normed input, made by the write before
+        (the embedding's, or the previous layer's last). st.next_reader: the next layer's (None: the last)."""
+        P = self.proj(st.h)
+        y = self.mixer.forward(st.h, P, self.cols, sv, cache)
+        _, out_w, mix = self.hc[0]
+        if self.ff is not None:
+            st.write(y, mix, out_w, (self.hc[1][0], self.norm2))
+            y = self.ff.forward(st.h, out_f32=True)
+            _, out_w, mix = self.hc[1]
+        st.write(y, mix, out_w, st.next_reader)
+
+
+ARRANGEMENTS = {"gated_parallel": GatedParallelLayer, "post_norm": PostNormLayer, "hyper_pre_norm": HyperPreNormLayer}
+
+
+class _HyperStream:
+    """The stream's copies of one step: ``xs`` fp32 [S, T, W], ``h`` the next sublayer's normed input in the
+    activation dtype, ``x`` (after the last layer's write) the sum of the copies."""
+
+    def __init__(self, S: int, T: int, W: int, act_dtype, device, keep_sums: bool):
+        self.xs = torch.empty(S, T, W, dtype=torch.float32, device=device)
+        self.h = torch.empty(T, W, dtype=act_dtype, device=device)
+        self.x = torch.empty(T, W, dtype=torch.float32, device=device)
+        self.next_reader, self.keep_sums = None, keep_sums
+
+    def write(self, y, mix, out_w, reader) -> None:
+        rd = {} if reader is None else dict(read_w=reader[0], alpha=reader[1].alpha, w=reader[1].w, b=reader[1].b, h_out=self.h)
+        last = reader is None or (self.keep_sums and reader is self.next_reader)
+        seq.hyper_mix(self.xs, y, mix, out_w, sum_out=self.x if last else None, **rd)
 
 
 class _Stream:
@@ -226,8 +320,10 @@ class HybridModel:
         # depth-average coefficients belong to the position in the stack, not to the (possibly shared) weights
         self.depth_coef = [_f32(tensors[f"l{i}.dwa"], self.device) for i in range(arch.num_layers)] \
             if arch.depth_average else None
-        self.scalar_norm = arch.arrangement != "post_norm"   # one number per norm, or a weight vector
-        self.final_norm = _f32(tensors["final.norm"].reshape(-1), self.device)
+        self.scalar_norm = arch.arrangement == "gated_parallel"   # one number per norm, or a weight vector
+        self.hyper = arch.arrangement == "hyper_pre_norm"
+        self.final_norm = _TanhNorm(tensors, "final.norm", self.device) if self.hyper else \
+            _f32(tensors["final.norm"].reshape(-1), self.device)
         self.head = Proj(tensors["head"], self.device, self.f32)
         self.capture_layers: list | None = None  # set to [] to record the residual stream after every layer
         self.last_resid = None
@@ -250,6 +346,9 @@ class HybridModel:
     def forward(self, sv, caches, part_size: int = 0, return_hidden: bool = False) -> torch.Tensor:
         """One step. Returns fp32 logits [S, vocab] of the sample rows, or with ``return_hidden`` the
         fp32 residual stream [T, width] after the last layer."""
+        if self.hyper:
+            x = self._forward_hyper(sv, caches)
+            return x if return_hidden else self._padded_logits(x, sv)
         T = sv.T
         W = self.arch.hidden_size
         dev, eps = self.device, self.arch.rms_eps
@@ -268,6 +367,28 @@ class HybridModel:
         self.last_resid = x
         if return_hidden:
             return x
+        return self._padded_logits(x, sv)
+
+    def _forward_hyper(self, sv, caches) -> torch.Tensor:
+        """The layer loop over several copies of the stream; returns their sum, fp32 [T, width]."""
+        S, T, W = self.arch.streams, sv.T, self.arch.hidden_size
+        st = _HyperStream(S, T, W, self.act_dtype, self.device, keep_sums=self.capture_layers is not None)
+        seq.embed_rows(sv.ids, self.embed, st.xs[0], prev=sv.prev_tokens)
+        for s in range(1, S):
+            st.xs[s].copy_(st.xs[0])
+        first = self.layers[0].reader()
+        st.next_reader = first
+        st.write(None, None, None, first)   # the first sublayer's input (nothing to add yet)
+        for li, L in enumerate(self.layers):
+            st.next_reader = self.layers[li + 1].reader() if li + 1 < len(self.layers) else None
+            L.run(st, sv, caches[li])
+            if self.capture_layers is not None:
+                self.capture_layers.append(st.x.clone())
+        self.last_resid = st.x
+        return st.x
+
+    def _padded_logits(self, x: torch.Tensor, sv) -> torch.Tensor:
+        dev = x.device
         V = self.arch.vocab_size
         if V % 4 == 0:
             return self.logits_of(x, sv.sample_idx)
@@ -279,7 +400,11 @@ class HybridModel:
     def logits_of(self, x: torch.Tensor, rows: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
         """fp32 logits [len(rows), vocab] of rows of the residual stream (final norm + head)."""
         hn = torch.empty(rows.numel(), x.shape[1], dtype=self.act_dtype, device=x.device)
-        seq.norm_rows(x, self.final_norm, self.arch.rms_eps, hn, rows=rows, scalar=self.scalar_norm)
+        if self.hyper:
+            n = self.final_norm
+            seq.tanh_norm_rows(x, n.alpha, n.w, n.b, hn, rows=rows)
+        else:
+            seq.norm_rows(x, self.final_norm, self.arch.rms_eps, hn, rows=rows, scalar=self.scalar_norm)
         return self.head(hn, out_f32=True, out=out)[:, : self.arch.vocab_size]
 
 
@@ -288,10 +413,14 @@ def tensor_shapes(arch: HybridArch, nominal: int | None = 16) -> dict:
     """name -> shape of every tensor of a checkpoint of ``arch`` (weight-owning layers only). A size
     that only a checkpoint's tensors give (a low-rank gate's width) is ``nominal``; None leaves it open."""
     W = arch.hidden_size
-    vector = arch.arrangement == "post_norm"
+    vector = arch.arrangement != "gated_parallel"
     out = {"embed": (arch.vocab_size, W), "final.norm": (W,) if vector else (), "head": (arch.vocab_size, W)}
+    extra = {}
+    if arch.arrangement == "hyper_pre_norm":
+        out.update(_TanhNorm.shapes("final.norm", W))
+        extra = {"streams": arch.streams}
     for i in sorted({arch.owner(i) for i in range(arch.num_layers)}):
-        out.update({f"l{i}.{k}": v for k, v in ARRANGEMENTS[arch.arrangement].shapes(arch.layers[i], W).items()})
+        out.update({f"l{i}.{k}": v for k, v in ARRANGEMENTS[arch.arrangement].shapes(arch.layers[i], W, **extra).items()})
     if arch.depth_average:
         out.update({f"l{i}.dwa": (i + 2,) for i in range(arch.num_layers)})
     return {k: tuple(nominal if d is None else d for d in v) for k, v in out.items()}
@@ -331,9 +460,20 @@ def random_tensors(arch: HybridArch, seed: int = 0) -> dict:
     out = {}
     for name, shape in tensor_shapes(arch).items():
         leaf = name.split(".")[-1] if not name.endswith(".b") else "b"
+        hyper = ".hc" in name
         if leaf == "dwa":  # close to "hand on the newest result"
             w = 0.1 * torch.randn(shape, generator=g) / shape[0]
             w[-1] += 1.0
+        elif hyper and leaf == "mix":    # close to "every copy keeps itself"
+            w = torch.eye(shape[0]) + 0.2 * torch.randn(shape, generator=g)
+        elif hyper and leaf == "in":
+            w = (1.0 + 0.3 * torch.randn(shape, generator=g)) / shape[0]
+        elif hyper and leaf == "out":
+            w = 1.0 + 0.3 * torch.randn(shape, generator=g)
+        elif leaf in ("alpha", "temp"):  # positive, near 1
+            w = 0.8 + 0.2 * torch.rand(shape, generator=g)
+        elif leaf in ("r1", "r2"):       # positive: ln(1 + r2 * distance) must exist
+            w = 0.05 + 0.5 * torch.rand(shape, generator=g)
         elif len(shape) == 2:
             std = 0.5 if name == "embed" else 1.0 / math.sqrt(shape[1])
             w = torch.randn(shape, generator=g) * std

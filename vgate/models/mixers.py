@@ -10,14 +10,17 @@ spec, so another design can reuse a mixer with other values.
   are absorbed into the query and the output.
 * :class:`GeneralDelta` — generalized delta rule with per-channel decay over an fp32 state matrix
   per head, kept in a state slot per sequence.
-* :class:`WindowAttention` — grouped-query attention over a sliding window of a paged key/value cache,
-  optionally with one mean key / value per block of tokens that has left the window, a sink in the
+* :class:`WindowAttention` — grouped-query attention over a sliding window (or all) of a paged key/value
+  cache, optionally with one mean key / value per block of tokens that has left the window, a sink in the
   softmax denominator, query / key norms over the head or the whole projection, values rotated by
-  their position.
+  their position, a bias on the scores that depends on the distance (logarithmic penalty or a learned
+  table over distance buckets), per-head and per-position query temperatures, a sigmoid output gate.
 * :class:`LinearAttention` — decayed outer-product recurrence S <- diag(a) S + k v^T, o = S^T q over an
-  fp32 state per head in a state slot; the decay is a constant per head or a gated value per key channel.
+  fp32 state per head in a state slot; the decay is a constant per head or a gated value per key channel;
+  optional rotary positions on q / k.
 * :class:`ParallelMixers` — two mixers reading the same input, their outputs added with fixed scales.
-* :class:`DenseFF`, :class:`MoEFF` — gated feed-forward; sigmoid-routed mixture of clamped gated experts.
+* :class:`DenseFF`, :class:`MoEFF` — gated feed-forward; mixture of gated experts (sigmoid scores with a
+  selection-only correction or softmax scores, clamped or SiLU experts, optional shared expert).
 """
 from __future__ import annotations
 
@@ -249,18 +252,30 @@ class WindowAttention:
     (the cached value of position j is turned by j in pairs over all of vdim, the attention output
     of position i is turned back by i), ``sink`` (one learned logit per head that only enters the
     softmax denominator), ``bias`` (q / k / v biases), ``out_bias``.
+    ``window`` None: every earlier position is seen. ``qk_norm_weight`` False: the head norm has no weight.
+    ``head_temp``: the scores of head h are multiplied by the tensor ``temp`` [h]. ``q_temp`` {coef, every}:
+    the query at position p is multiplied by 1 + coef ln(floor((p + 1) / every) + 1). ``dist_bias``: a term
+    of the score that depends on the head and the distance n = i - j alone, {"kind": "log"}:
+    -r1[h] ln(1 + r2[h] n) (tensors ``r1``, ``r2``); {"kind": "table", "far": F}: rel[bucket(n), h] with the
+    learned tensor ``rel`` [B, heads], bucket(n) = n below B/2 and log-spaced rows from B/2 to F above
+    (:func:`distance_buckets`). ``gate`` "sigmoid": the heads' outputs are multiplied by sigmoid(W_g h)
+    before the output projection.
     """
     kind = "window_attention"
     cache = "paged"
+    FULL = 1 << 30   # "window" of a layer that sees every earlier position
 
     def __init__(self, spec: dict, width: int, eps: float, tensors: dict, device, f32: bool):
         m = spec
         self.H, self.G, self.D, self.V = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
         if self.G < 1 or self.H % self.G:
             raise ValueError("window_attention: heads must be a multiple of kv_heads")
-        self.scale, self.window, self.pool = float(m["scale"]), int(m["window"]), int(m.get("pool") or 0)
-        if self.window < 1 or self.pool < 0:
+        self.scale, self.pool = float(m["scale"]), int(m.get("pool") or 0)
+        self.window = self.FULL if m.get("window") is None else int(m["window"])
+        if self.window < 1 or self.pool < 0 or self.window > self.FULL:
             raise ValueError("window_attention: window >= 1, pool >= 0")
+        if self.pool and m.get("window") is None:
+            raise ValueError("window_attention: pooled blocks need a window")
         self.qk_norm = m.get("qk_norm", "none")
         if self.qk_norm not in ("none", "head", "all"):
             raise ValueError(f"window_attention: qk_norm {self.qk_norm!r}")
@@ -274,12 +289,40 @@ class WindowAttention:
         base = float(rot.get("base", 10000.0))
         self.inv_freq = seq.rope_inv_freq(dims, base, dev, scaling=rot.get("scaling"))
         self.v_freq = seq.rope_inv_freq(self.V, base, dev) if m.get("rotate_values") else None
-        self.in_rows = [(n, tensors[n]) for n in ("q", "k", "v")]
+        self.gated = m.get("gate") == "sigmoid"
+        if m.get("gate") not in (None, "sigmoid"):
+            raise ValueError(f"window_attention: gate {m.get('gate')!r}")
+        self.in_rows = [(n, tensors[n]) for n in ("q", "k", "v") + (("g",) if self.gated else ())]
         self.in_bias = {n: tensors[n + ".b"] for n in ("q", "k", "v")} if m.get("bias") else {}
         self.qw = self.kw = None
         if self.qk_norm != "none":
-            self.qw, self.kw = _f32(tensors["q.norm"], dev), _f32(tensors["k.norm"], dev)
+            if m.get("qk_norm_weight", True):
+                self.qw, self.kw = _f32(tensors["q.norm"], dev), _f32(tensors["k.norm"], dev)
+            else:
+                n = self.D if self.qk_norm == "head" else None
+                self.qw = torch.ones(n or self.H * self.D, dtype=torch.float32, device=dev)
+                self.kw = torch.ones(n or self.G * self.D, dtype=torch.float32, device=dev)
         self.sink = _f32(tensors["sink"], dev) if m.get("sink") else None
+        self.head_temp = _f32(tensors["temp"], dev) if m.get("head_temp") else None
+        qt = m.get("q_temp") or {}
+        self.q_temp = (float(qt.get("coef", 0.0)), int(qt.get("every", 1)))
+        if self.q_temp[1] < 1:
+            raise ValueError("window_attention: q_temp.every >= 1")
+        db = m.get("dist_bias") or {}
+        self.bias_kind, self.bias_a, self.bias_b = seq.BIAS_NONE, None, None
+        if db.get("kind") == "log":
+            self.bias_kind, self.bias_a, self.bias_b = seq.BIAS_LOG, _f32(tensors["r1"], dev), _f32(tensors["r2"], dev)
+        elif db.get("kind") == "table":
+            rel = tensors["rel"].float()
+            rows = distance_buckets(rel.shape[0], float(db["far"]))
+            # expanded once to one entry per distance (the last stands for every larger one), head-major
+            self.bias_kind, self.bias_a = seq.BIAS_TABLE, rel[torch.tensor(rows)].t().contiguous().to(dev)
+            if rel.shape[1] != self.H:
+                raise ValueError("window_attention: the distance table needs one column per head")
+        elif db:
+            raise ValueError(f"window_attention: dist_bias kind {db.get('kind')!r}")
+        if self.bias_kind and self.pool:
+            raise ValueError("window_attention: a distance bias and pooled blocks do not combine")
         self.o = Proj(tensors["o"], dev, f32, bias=tensors["o.b"] if m.get("out_bias") else None)
 
     @staticmethod
@@ -288,10 +331,21 @@ class WindowAttention:
         out = {"q": (H * D, width), "k": (G * D, width), "v": (G * V, width), "o": (width, H * V)}
         if spec.get("bias"):
             out.update({"q.b": (H * D,), "k.b": (G * D,), "v.b": (G * V,)})
-        if spec.get("qk_norm", "none") == "head":
+        if not spec.get("qk_norm_weight", True):
+            pass
+        elif spec.get("qk_norm", "none") == "head":
             out.update({"q.norm": (D,), "k.norm": (D,)})
         elif spec.get("qk_norm") == "all":
             out.update({"q.norm": (H * D,), "k.norm": (G * D,)})
+        if spec.get("gate"):
+            out["g"] = (H * V, width)
+        if spec.get("head_temp"):
+            out["temp"] = (H,)
+        kind = (spec.get("dist_bias") or {}).get("kind")
+        if kind == "log":
+            out.update({"r1": (H,), "r2": (H,)})
+        elif kind == "table":   # None: the number of buckets, which only the tensor gives
+            out["rel"] = (None, H)
         if spec.get("sink"):
             out["sink"] = (H,)
         if spec.get("out_bias"):
@@ -327,14 +381,31 @@ class WindowAttention:
         kc, vc, kp, vp, vt = cache
         q = torch.empty(T, self.H * self.D, dtype=h.dtype, device=h.device)
         seq.window_write(cols(P, "q"), cols(P, "k"), cols(P, "v"), self.qw, self.kw, self.eps, self.qk_norm == "all",
-                         sv.positions, sv.slots, self.inv_freq, self.rot_dims, self.v_freq, kc, vc, q, self.H, self.G, vt=vt)
+                         sv.positions, sv.slots, self.inv_freq, self.rot_dims, self.v_freq, kc, vc, q, self.H, self.G, vt=vt,
+                         q_head_scale=self.head_temp, q_temp_coef=self.q_temp[0], q_temp_every=self.q_temp[1])
         if self.pool:
             seq.window_pool(kc, vc, kp, vp, sv.positions, sv.block_tables, sv.query_start, self.pool,
                             num_seqs=sv.num_seqs or None)
         o = torch.empty(T, self.H * self.V, dtype=h.dtype, device=h.device)
         seq.window_attn(q, kc, vc, kp, vp, sv.block_tables, sv.context_lens, sv.query_start, o, self.scale, self.H,
-                        self.window, self.pool, self.sink, self.v_freq, num_seqs=sv.num_seqs or None, vt=vt)
+                        self.window, self.pool, self.sink, self.v_freq, num_seqs=sv.num_seqs or None, vt=vt,
+                        bias_kind=self.bias_kind, bias_a=self.bias_a, bias_b=self.bias_b,
+                        gate=cols(P, "g") if self.gated else None)
         return self.o(o, out_f32=True)
+
+
+def distance_buckets(B: int, far: float) -> list:
+    """Row of a [B, heads] distance table for every distance 0 .. ceil(far): distances below B // 2 have a
+    row each, the rows from B // 2 on are spaced evenly in ln(distance) between B // 2 and ``far``, and the
+    last row takes everything beyond (so the list's last entry stands for all larger distances)."""
+    half = B // 2
+    if half < 1 or far <= half:
+        raise ValueError("distance table: at least two rows, and far > rows / 2")
+    rows = []
+    for n in range(max(int(math.ceil(far)), half) + 1):
+        rows.append(n if n < half else
+                    min(B - 1, half + int(math.floor(math.log(n / half) / math.log(far / half) * (B - half)))))
+    return rows
 
 
 class LinearAttention:
@@ -345,8 +416,11 @@ class LinearAttention:
     {"kind": "channel", "tau": tau}: a = sigmoid(z)^(1 / tau) per key channel with z = W_a2 (W_a1 h) +
     b, a low-rank gate whose width the checkpoint's tensors give), ``q_scale``, ``in_act`` ("none" |
     "silu" on q, k and v), ``out_norm`` ("head": RMS norm per head with one [vdim] weight | "all":
-    over the concatenated heads with a [heads * vdim] weight), ``gate_act`` ("silu" | "sigmoid" of
-    W_g h, multiplied onto the normed output before the output projection).
+    over the concatenated heads with a [heads * vdim] weight; ``norm_weight`` False: no weight),
+    ``gate_act`` ("silu" | "sigmoid" of W_g h, multiplied onto the normed output before the output
+    projection), ``rot`` {dims, base, layout "half" | "pairs"}: rotary positions on the first ``dims``
+    entries of every q / k head (entry i paired with i + dims / 2, or 2i with 2i + 1), ``k_scale``
+    (keys multiplied after the rotation).
     """
     kind = "linear_attention"
     cache = "state"
@@ -364,7 +438,13 @@ class LinearAttention:
         for key, allowed in (("in_act", ("none", "silu")), ("out_norm", ("head", "all")), ("gate_act", ("silu", "sigmoid"))):
             if spec[key] not in allowed:
                 raise ValueError(f"linear_attention: {key} {spec[key]!r}")
-        self.q_scale = float(spec.get("q_scale", 1.0))
+        self.q_scale, self.k_scale = float(spec.get("q_scale", 1.0)), float(spec.get("k_scale", 1.0))
+        rot = spec.get("rot") or {}
+        dims = int(rot.get("dims", 0))
+        if dims > self.D or dims < 0 or rot.get("layout", "half") not in ("half", "pairs"):
+            raise ValueError("linear_attention: rot.dims <= dim, layout half | pairs")
+        self.rot_dims, self.rot_half = 2 * (dims // 2), rot.get("layout", "half") == "half"
+        self.inv_freq = seq.rope_inv_freq(dims, float(rot.get("base", 10000.0)), dev) if self.rot_dims else None
         self.in_silu, self.norm_all, self.gate_silu = spec["in_act"] == "silu", spec["out_norm"] == "all", spec["gate_act"] == "silu"
         self.in_rows = [(n, tensors[n]) for n in ("q", "k", "v", "g")]
         self.in_bias = {}
@@ -377,14 +457,15 @@ class LinearAttention:
             self.a2 = Proj(tensors["a2"], dev, f32, allow_packed=False, bias=tensors["a2.b"])  # fp32 gate logits
         else:
             self.head_decay = torch.tensor([float(d) for d in dec["values"]], dtype=torch.float32, device=dev)
-        self.nw = _f32(tensors["norm"], dev)
+        self.nw = _f32(tensors["norm"], dev) if spec.get("norm_weight", True) else None
         self.o = Proj(tensors["o"], dev, f32)
 
     @staticmethod
     def shapes(spec: dict, width: int) -> dict:
         H, D, V = spec["heads"], spec["dim"], spec["vdim"]
-        out = {"q": (H * D, width), "k": (H * D, width), "v": (H * V, width), "g": (H * V, width), "o": (width, H * V),
-               "norm": (H * V,) if spec["out_norm"] == "all" else (V,)}
+        out = {"q": (H * D, width), "k": (H * D, width), "v": (H * V, width), "g": (H * V, width), "o": (width, H * V)}
+        if spec.get("norm_weight", True):
+            out["norm"] = (H * V,) if spec["out_norm"] == "all" else (V,)
         if spec["decay"]["kind"] == "channel":  # None: the gate's width, which only the tensors give
             out.update({"a1": (None, width), "a2": (H * D, None), "a2.b": (H * D,)})
         return out
@@ -404,7 +485,8 @@ class LinearAttention:
         out = torch.empty(T, self.H * self.V, dtype=h.dtype, device=h.device)
         seq.linear_attn(cols(P, "q"), cols(P, "k"), cols(P, "v"), cols(P, "g"), z, self.head_decay, self.tau, self.q_scale,
                         self.in_silu, self.nw, self.norm_all, self.gate_silu, cache, sv.state_slots, sv.context_lens,
-                        sv.query_start, out, self.eps, num_seqs=sv.num_seqs or None)
+                        sv.query_start, out, self.eps, num_seqs=sv.num_seqs or None, k_scale=self.k_scale,
+                        positions=sv.positions, inv_freq=self.inv_freq, rot_dims=self.rot_dims, rot_half=self.rot_half)
         return self.o(out, out_f32=True)
 
 
@@ -478,52 +560,68 @@ class DenseFF:
 
 
 class MoEFF:
-    """Sigmoid-routed experts: the ``top`` largest of sigmoid(z) + correction are chosen, weighted by
-    their uncorrected scores over the sum. Expert: g = min(gate h, L), u = clamp(up h, -L, L),
-    down(g * sigmoid(alpha g) * (u + 1))."""
+    """Routed experts: scores s = sigmoid(z) or softmax(z) over all experts (``router.score``, fp32); the
+    ``top`` largest of s (+ a selection-only ``correction`` tensor unless ``router.correction`` is False)
+    are chosen, weighted by their scores over the chosen scores' sum, times ``router.scale``. Expert
+    (``expert.act``): "clamped": g = min(gate h, L), u = clamp(up h, -L, L), down(g * sigmoid(alpha g) * (u + 1));
+    "silu": down(silu(gate h) * (up h)). ``shared`` {ff}: a dense gated expert every token runs, added."""
     ALPHA = 1.702
     SUM_EPS = 1e-20
 
     def __init__(self, spec: dict, width: int, tensors: dict, device, f32: bool):
-        self.E, self.top = int(spec["router"]["experts"]), int(spec["router"]["top"])
-        self.ff, self.limit = int(spec["expert"]["ff"]), float(spec["expert"]["limit"])
+        r = spec["router"]
+        self.E, self.top = int(r["experts"]), int(r["top"])
+        self.ff = int(spec["expert"]["ff"])
+        self.act = {"clamped": seq.ACT_CLAMPED_GLU, "silu": seq.ACT_SILU_MUL}[spec["expert"].get("act", "clamped")]
+        self.limit = float(spec["expert"]["limit"]) if self.act == seq.ACT_CLAMPED_GLU else 0.0
+        self.softmax = {"sigmoid": False, "softmax": True}[r.get("score", "sigmoid")]
+        self.scale = float(r.get("scale", 1.0))
         dev = torch.device(device)
         dt = torch.float32 if f32 else torch.bfloat16
         self.f32 = f32
         self.router = Proj(tensors["router"], dev, f32, allow_packed=False)  # fp32 logits, N = experts
-        self.corr = _f32(tensors["correction"], dev)
+        self.corr = _f32(tensors["correction"], dev) if r.get("correction", True) else None
         st = lambda n: torch.stack([tensors[f"e{e}.{n}"] for e in range(self.E)]).to(dev, dt).contiguous()  # noqa: E731
         self.gate, self.up, self.down = st("gate"), st("up"), st("down")
+        self.shared = None
+        if spec.get("shared"):
+            sh = {k[len("shared."):]: v for k, v in tensors.items() if k.startswith("shared.")}
+            self.shared = DenseFF({"ff": int(spec["shared"]["ff"]), "act": spec["shared"].get("act", "silu")}, width, sh, dev, f32)
 
     @staticmethod
     def shapes(spec: dict, width: int) -> dict:
         E, ff = spec["router"]["experts"], spec["expert"]["ff"]
-        out = {"router": (E, width), "correction": (E,)}
+        out = {"router": (E, width)}
+        if spec["router"].get("correction", True):
+            out["correction"] = (E,)
         for e in range(E):
             out.update({f"e{e}.gate": (ff, width), f"e{e}.up": (ff, width), f"e{e}.down": (width, ff)})
+        if spec.get("shared"):
+            out.update({"shared." + k: v for k, v in DenseFF.shapes(spec["shared"], width).items()})
         return out
 
     def nbytes(self) -> int:
-        return self.router.nbytes() + 3 * self.gate.numel() * self.gate.element_size()
+        return (self.router.nbytes() + 3 * self.gate.numel() * self.gate.element_size()
+                + (self.shared.nbytes() if self.shared else 0))
 
-    def forward(self, h: torch.Tensor) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, out_f32: bool = False) -> torch.Tensor:
         T, W = h.shape
         dev, dt = h.device, h.dtype
         z = self.router(h, out_f32=True)
         idx = torch.empty(T, self.top, dtype=torch.int32, device=dev)
         wts = torch.empty(T, self.top, dtype=torch.float32, device=dev)
-        seq.moe_route(z, self.corr, self.top, self.SUM_EPS, idx, wts)
+        seq.moe_route(z, self.corr, self.top, self.SUM_EPS, idx, wts, softmax=self.softmax, scale=self.scale)
         rows = torch.empty(T * self.top, dtype=torch.int32, device=dev)
         pos = torch.empty(T * self.top, dtype=torch.int32, device=dev)
         off = torch.empty(self.E + 1, dtype=torch.int32, device=dev)
         seq.moe_sort(idx, self.E, rows, pos, off)
         a1 = torch.empty(T * self.top, self.ff, dtype=dt, device=dev)
-        seq.gemm(h, self.gate, a1, w2=self.up, a_rows=rows, group_off=off, act=seq.ACT_CLAMPED_GLU, limit=self.limit,
+        seq.gemm(h, self.gate, a1, w2=self.up, a_rows=rows, group_off=off, act=self.act, limit=self.limit,
                  alpha=self.ALPHA)
         y = torch.empty(T * self.top, W, dtype=dt, device=dev)
         seq.gemm(a1, self.down, y, group_off=off)
-        out = torch.empty(T, W, dtype=dt, device=dev)
-        seq.moe_combine(y, pos, wts, out)
+        out = torch.empty(T, W, dtype=torch.float32 if out_f32 else dt, device=dev)
+        seq.moe_combine(y, pos, wts, out, add=self.shared.forward(h, out_f32=out_f32) if self.shared else None)
         return out
 
 

@@ -43,6 +43,8 @@ def _C():
 
 
 ACT_NONE, ACT_SILU_MUL, ACT_CLAMPED_GLU, ACT_TANH, ACT_GELU_TANH_MUL = 0, 1, 2, 3, 4
+BIAS_NONE, BIAS_LOG, BIAS_TABLE = 0, 1, 2   # distance term of an attention score (see window_attn)
+MAX_STREAMS = 8             # copies of the residual stream hyper_mix takes
 LINEAR_ATTN_MAX_DIM = 256   # key channels per head the recurrence kernel keeps in registers (csrc/kernels/linear_attn.hip)
 
 
@@ -171,6 +173,21 @@ def _rope_pairs(x: torch.Tensor, pos: torch.Tensor, inv_freq: torch.Tensor, dims
     return y
 
 
+def _rope_halves(x: torch.Tensor, pos: torch.Tensor, inv_freq: torch.Tensor, dims: int) -> torch.Tensor:
+    """Rotate the leading ``dims`` entries of the last axis, entry i paired with entry i + dims / 2; fp32."""
+    y = x.clone()
+    if dims == 0:
+        return y
+    half = dims // 2
+    ang = pos.float()[:, None] * inv_freq[None, :half]
+    shape = [x.shape[0]] + [1] * (x.dim() - 2) + [half]
+    c, s = torch.cos(ang).view(shape), torch.sin(ang).view(shape)
+    u, v = x[..., :half], x[..., half:dims]
+    y[..., :half] = u * c - v * s
+    y[..., half:dims] = v * c + u * s
+    return y
+
+
 def latent_write(kv, w, eps, positions, slots, inv_freq, rot_dims: int, cache, rank: int, cache_t=None) -> None:
     """cache[slot] = [rmsnorm(kv[:rank]) * w, rope(kv[rank:])] for every token with slot >= 0.
     ``cache_t`` (GPU, bf16): a second copy of the latent part laid out [page, column, key in page], the
@@ -258,12 +275,13 @@ def delta_rule(r, k, v, g, a, wl, w0, ab, nw, state, state_slots, context_lens, 
         state[slot] = St
 
 
-def moe_route(z, corr, top: int, norm_eps: float, idx, wts) -> None:
-    """idx / wts [T, top]: largest sigmoid(z) + corr; weights sigmoid(z) of the chosen over their sum."""
+def moe_route(z, corr, top: int, norm_eps: float, idx, wts, softmax: bool = False, scale: float = 1.0) -> None:
+    """idx / wts [T, top]: the ``top`` largest of s + corr with s = sigmoid(z), or softmax(z) over all
+    experts; weights s of the chosen over (their sum + norm_eps), times ``scale``."""
     if z.is_cuda:
-        _C().moe_route(z, corr, top, norm_eps, idx, wts)
+        _C().moe_route(z, corr, top, norm_eps, idx, wts, softmax, scale)
         return
-    s = torch.sigmoid(z)
+    s = torch.softmax(z, -1) if softmax else torch.sigmoid(z)
     choice = s + corr if corr is not None else s
     # arg-max rounds, lowest index first on ties (the kernel's order)
     c = choice.clone()
@@ -275,7 +293,7 @@ def moe_route(z, corr, top: int, norm_eps: float, idx, wts) -> None:
     ii = torch.stack(picks, 1)
     ws = torch.gather(s, 1, ii)
     idx.copy_(ii.int())
-    wts.copy_(ws / (ws.sum(-1, keepdim=True) + norm_eps))
+    wts.copy_(ws / (ws.sum(-1, keepdim=True) + norm_eps) * scale)
 
 
 def moe_sort(idx, E: int, rows, pos, off) -> None:
@@ -294,14 +312,15 @@ def moe_sort(idx, E: int, rows, pos, off) -> None:
     off.copy_(torch.cat([torch.zeros(1, dtype=torch.long), cnt.cumsum(0)]).int())
 
 
-def moe_combine(y, pos, wts, out) -> None:
-    """out[t] = sum_c wts[t, c] * y[pos[t, c]]."""
+def moe_combine(y, pos, wts, out, add=None) -> None:
+    """out[t] = sum_c wts[t, c] * y[pos[t, c]] [+ add[t]] (fp32 sum; out bf16 or fp32)."""
     if y.is_cuda:
-        _C().moe_combine(y, pos, wts, out)
+        _C().moe_combine(y, pos, wts, out, add)
         return
     T, top = wts.shape
     rows = y.float()[pos.view(T, top).long()]
-    out.copy_((rows * wts[:, :, None]).sum(1))
+    r = (rows * wts[:, :, None]).sum(1)
+    out.copy_(r if add is None else r + add[:T].float())
 
 
 # ------------------------------------------------------------------ post-norm residual, depth average
@@ -312,6 +331,42 @@ def cast_rows(x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
         return out
     out.copy_(x[: out.shape[0]])
     return out
+
+
+def tanh_norm_rows(x: torch.Tensor, alpha: torch.Tensor, w: torch.Tensor, b: torch.Tensor, out: torch.Tensor,
+                   rows: torch.Tensor | None = None) -> torch.Tensor:
+    """out[m] = tanh(alpha * x[rows[m]]) * w + b: a norm without statistics (alpha one fp32 number, w / b
+    fp32 vectors), computed in fp32 and rounded to out's dtype."""
+    if x.is_cuda:
+        _C().tanh_norm_rows(x, alpha, w, b, out, rows)
+        return out
+    xf = x.float()
+    xf = xf[rows.long()] if rows is not None else xf[: out.shape[0]]
+    out.copy_(torch.tanh(alpha * xf) * w + b)
+    return out
+
+
+def hyper_mix(xs: torch.Tensor, y: torch.Tensor | None, mix: torch.Tensor | None, out_w: torch.Tensor | None,
+              read_w: torch.Tensor | None = None, alpha=None, w=None, b=None, h_out: torch.Tensor | None = None,
+              sum_out: torch.Tensor | None = None) -> None:
+    """One sublayer's write to ``xs`` [S, T, W] (fp32 copies of the residual stream), fused with the next
+    sublayer's read. With ``y`` [T, W]: all copies at once from the old ones,
+        xs[t] <- sum_s mix[s, t] xs[s] + out_w[t] * y.
+    With ``read_w`` [S]: u = sum_s read_w[s] xs[s] (the new copies), h_out = tanh(alpha u) * w + b in h_out's
+    dtype. With ``sum_out`` [T, W] fp32: the sum of the (new) copies. Everything in fp32."""
+    if xs.is_cuda:
+        _C().hyper_mix(xs, y, mix, out_w, read_w, alpha, w, b, h_out, sum_out)
+        return
+    if y is not None:
+        T = y.shape[0]
+        new = torch.einsum("st,snw->tnw", mix, xs[:, :T]) + out_w[:, None, None] * y.float()[None]
+        xs[:, :T] = new
+    if read_w is not None:
+        T = h_out.shape[0]
+        u = torch.einsum("s,snw->nw", read_w, xs[:, :T])
+        h_out.copy_(torch.tanh(alpha * u) * w + b)
+    if sum_out is not None:
+        sum_out.copy_(xs[:, : sum_out.shape[0]].sum(0))
 
 
 def glu_rows(gu: torch.Tensor, out: torch.Tensor, act: int) -> torch.Tensor:
@@ -356,17 +411,20 @@ def _rope_pairs_heads(x: torch.Tensor, pos: torch.Tensor, inv_freq: torch.Tensor
 
 
 def window_write(q, k, v, qw, kw, eps: float, norm_all: bool, positions, slots, inv_freq, rot_dims: int, v_freq,
-                 kc, vc, q_out, H: int, G: int, vt=None) -> None:
+                 kc, vc, q_out, H: int, G: int, vt=None, q_head_scale=None, q_temp_coef: float = 0.0,
+                 q_temp_every: int = 1) -> None:
     """Prepare one step's queries, keys and values of a window-attention layer.
     q [T, H * D], k [T, G * D], v [T, G * V] (biases already added). Query / key RMS norm (``qw`` / ``kw``
     None: none; ``norm_all``: over the whole projection with a [heads * D] weight, else per head with a
     [D] weight), rotation of the first ``rot_dims`` entries of every head, values turned over all of V
-    by ``v_freq`` if given. q goes to ``q_out``; keys and values to the paged caches
+    by ``v_freq`` if given. Query temperatures (fp32, after the norm): head h times ``q_head_scale`` [h], the
+    query at position p times 1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1). q goes to ``q_out``; keys and values to the paged caches
     kc [pages, G, page, D] / vc [pages, G, page, V] at the tokens' slots (slot < 0: padding row).
     ``vt`` (GPU, bf16): a second copy of the values laid out [pages, G, V, page], the operand layout of
     the MFMA attention kernel's weighted sum."""
     if q.is_cuda:
-        _C().window_write(q, k, v, qw, kw, eps, norm_all, positions, slots, inv_freq, rot_dims, v_freq, kc, vc, q_out, H, G, vt)
+        _C().window_write(q, k, v, qw, kw, eps, norm_all, positions, slots, inv_freq, rot_dims, v_freq, kc, vc, q_out, H, G, vt,
+                          q_head_scale, q_temp_coef, q_temp_every)
         return
     T = q.shape[0]
     D, V, page = kc.shape[3], vc.shape[3], kc.shape[2]
@@ -381,6 +439,11 @@ def window_write(q, k, v, qw, kw, eps: float, norm_all: bool, positions, slots, 
         return x * (1.0 / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps)) * w
 
     qn = _rope_pairs_heads(norm(qf, qw, H), positions[:T], inv_freq, rot_dims)
+    if q_head_scale is not None:
+        qn = qn * q_head_scale.view(1, H, 1)
+    if q_temp_coef != 0.0:
+        grow = 1.0 + q_temp_coef * torch.log(torch.floor((positions[:T] + 1).float() / q_temp_every) + 1.0)
+        qn = qn * grow.view(T, 1, 1)
     kn = _rope_pairs_heads(norm(kf, kw, G), positions[:T], inv_freq, rot_dims)
     vn = vf.view(T, G, V)
     if v_freq is not None:
@@ -417,17 +480,21 @@ def window_pool(kc, vc, kp, vp, positions, block_tables, query_start, pool: int,
 
 
 def window_attn(q, kc, vc, kp, vp, block_tables, context_lens, query_start, out, scale: float, H: int, window: int,
-                pool: int, sink, v_freq, num_seqs: int | None = None, vt=None, prefill_kernel: int = 0) -> None:
+                pool: int, sink, v_freq, num_seqs: int | None = None, vt=None, prefill_kernel: int = 0,
+                bias_kind: int = BIAS_NONE, bias_a=None, bias_b=None, gate=None) -> None:
     """out[t, h] = sum_j p_j value_j over the keys position i of token t sees: the tokens j with
     0 <= i - j < window and, with ``pool`` = P > 0, the pooled row of every block b with
     b P + P - 1 <= i - window; p = softmax(scale q . key) over both kinds together, with exp(sink[h]) added
     to the denominator if ``sink`` is given. With ``v_freq`` the result is turned back by -i over all of V.
-    Query head h reads key/value head h / (H / G). With ``vt`` (see :func:`window_write`) bf16 caches run
+    Query head h reads key/value head h / (H / G). A distance term (no pooled blocks then) is added to the
+    scaled score of the token at distance n = i - j: ``BIAS_LOG``: -bias_a[h] * ln(1 + bias_b[h] * n);
+    ``BIAS_TABLE``: bias_a[h, min(n, last)] (fp32 [H, distances]). ``gate`` [T, H * V]: the result is
+    multiplied by sigmoid(gate). With ``vt`` (see :func:`window_write`) bf16 caches run
     the MFMA kernels (``prefill_kernel``: which one prompt portions take, 0 = tiles staged in LDS for 64 rows,
     1 = 16 rows per workgroup with the tiles shared out over its waves)."""
     if q.is_cuda:
         _C().window_attn(q, kc, vc, kp, vp, block_tables, context_lens, query_start, out, scale, H, window, pool, sink, v_freq, vt,
-                         prefill_kernel)
+                         prefill_kernel, bias_kind, bias_a, bias_b, gate)
         return
     G, page, D, V = kc.shape[1], kc.shape[2], kc.shape[3], vc.shape[3]
     rep = H // G
@@ -451,23 +518,36 @@ def window_attn(q, kc, vc, kp, vp, block_tables, context_lens, query_start, out,
                 Vv = torch.cat([vp[pg, :, r // pool].float(), Vv])
             qh = q[t].float().view(G, rep, D)
             sc = torch.einsum("grd,ngd->grn", qh, K) * scale               # [G, rep, n]
+            if bias_kind != BIAS_NONE:
+                dist = (i - torch.arange(lo, i + 1))
+                if bias_kind == BIAS_LOG:
+                    bias = -bias_a.view(H, 1) * torch.log(1.0 + bias_b.view(H, 1) * dist.float())
+                else:
+                    bias = bias_a[:, dist.clamp(max=bias_a.shape[1] - 1)]
+                sc = sc + bias.view(G, rep, -1)
             if sink is not None:
                 sc = torch.cat([sc, sink.view(G, rep, 1)], -1)
             p = torch.softmax(sc, -1)[..., : K.shape[0]]
             o = torch.einsum("grn,ngv->grv", p, Vv).reshape(1, H, V)
             if v_freq is not None:
                 o = _rope_pairs(o, torch.tensor([-float(i)]), v_freq, 2 * v_freq.numel())
-            out[t] = o.reshape(H * V).to(out.dtype)
+            o = o.reshape(H * V)
+            if gate is not None:
+                o = o * torch.sigmoid(gate[t].float())
+            out[t] = o.to(out.dtype)
 
 
 # ---------------------------------------------------------------------------------- linear attention
 def linear_attn(q, k, v, g, z, head_decay, tau: float, q_scale: float, in_silu: bool, nw, norm_all: bool,
                 gate_silu: bool, state, state_slots, context_lens, query_start, out, eps: float,
-                num_seqs: int | None = None, cols_per_lane: int = 0) -> None:
+                num_seqs: int | None = None, cols_per_lane: int = 0, k_scale: float = 1.0, positions=None, inv_freq=None,
+                rot_dims: int = 0, rot_half: bool = True) -> None:
     """Decayed outer-product recurrence over state slots, state [slots, H, D, V] fp32:
         S <- diag(a_t) S + k_t v_t^T,  o_t = S^T (q_scale q_t)
     a_t = sigmoid(z_t)^(1 / tau) per key channel (``z`` fp32 [T, H * D]) or the constant head_decay[h];
-    ``in_silu``: silu on q, k, v. Then RMS norm of o (per head with a [V] weight, or with ``norm_all`` over
+    ``in_silu``: silu on q, k, v. With ``rot_dims`` > 0 the first rot_dims entries of every q / k head are
+    turned by position * inv_freq (``rot_half``: entry i with i + rot_dims / 2, else 2i with 2i + 1), then k is
+    multiplied by ``k_scale``. Then RMS norm of o (``nw`` None: no weight) (per head with a [V] weight, or with ``norm_all`` over
     the concatenated heads with a [H * V] weight), times silu(g) or sigmoid(g). A portion that starts at
     position 0 starts from a zero state. ``cols_per_lane`` (GPU): value columns a lane of the scan keeps, 0 =
     chosen by the launch's size."""
@@ -476,7 +556,8 @@ def linear_attn(q, k, v, g, z, head_decay, tau: float, q_scale: float, in_silu: 
         n = _C().linear_attn_scratch(q.shape[0], state_slots.numel(), H, D, V)
         scratch = torch.empty(n, dtype=torch.float32, device=q.device)
         _C().linear_attn(q, k, v, g, z, head_decay, tau, q_scale, in_silu, nw, norm_all, gate_silu, state, state_slots,
-                         context_lens, query_start, out, eps, scratch, cols_per_lane)
+                         context_lens, query_start, out, eps, scratch, cols_per_lane, k_scale, positions, inv_freq,
+                         rot_dims, rot_half)
         return
     H, D, V = state.shape[1], state.shape[2], state.shape[3]
     S = state_slots.numel() if num_seqs is None else num_seqs
@@ -489,8 +570,12 @@ def linear_attn(q, k, v, g, z, head_decay, tau: float, q_scale: float, in_silu: 
         n = t1 - t0
         pos0 = int(context_lens[s]) - n
         St = state[slot].clone() if pos0 > 0 else torch.zeros(H, D, V)
-        qq = act(q[t0:t1].float()).view(n, H, D) * q_scale
+        qq = act(q[t0:t1].float()).view(n, H, D)
         kk = act(k[t0:t1].float()).view(n, H, D)
+        if rot_dims:
+            turn = _rope_halves if rot_half else _rope_pairs
+            qq, kk = turn(qq, positions[t0:t1], inv_freq, rot_dims), turn(kk, positions[t0:t1], inv_freq, rot_dims)
+        qq, kk = qq * q_scale, kk * k_scale
         vv = act(v[t0:t1].float()).view(n, H, V)
         if z is not None:
             a = torch.exp(torch.nn.functional.logsigmoid(z[t0:t1].float()) / tau).view(n, H, D)
@@ -501,11 +586,12 @@ def linear_attn(q, k, v, g, z, head_decay, tau: float, q_scale: float, in_silu: 
             St = a[i][:, :, None] * St + kk[i][:, :, None] * vv[i][:, None, :]
             o[i] = torch.einsum("hdv,hd->hv", St, qq[i])
         state[slot] = St
+        one = 1.0 if nw is None else nw
         if norm_all:
             of = o.reshape(n, H * V)
-            of = of * (1.0 / torch.sqrt(of.pow(2).mean(-1, keepdim=True) + eps)) * nw
+            of = of * (1.0 / torch.sqrt(of.pow(2).mean(-1, keepdim=True) + eps)) * one
         else:
-            of = (o * (1.0 / torch.sqrt(o.pow(2).mean(-1, keepdim=True) + eps)) * nw).reshape(n, H * V)
+            of = (o * (1.0 / torch.sqrt(o.pow(2).mean(-1, keepdim=True) + eps)) * one).reshape(n, H * V)
         gg = g[t0:t1].float()
         of = of * (torch.nn.functional.silu(gg) if gate_silu else torch.sigmoid(gg))
         out[t0:t1] = of.to(out.dtype)
