@@ -2,9 +2,11 @@
 // slot between steps,
 //   S <- diag(a_t) S + k_t v_t^T,   o_t = S^T (q_scale q_t)
 // with a_t either a constant per head or sigmoid(z_t)^(1 / tau) per key channel (z fp32), optionally
-// silu on q, k and v, then an RMS norm of o (per head, or over the concatenated heads) and an output
-// gate silu(g) or sigmoid(g). Key and value sizes may differ. Three launches:
-//   prep   (token, head) parallel: the fp32 per-channel triples {a, k, q_scale q} and the values.
+// silu on q, k and v, optionally rotary positions on the leading rot_dims entries of every q / k head
+// (entry i paired with i + rot_dims / 2, or 2i with 2i + 1; angle = position * inv_freq in fp32) and a key
+// scale after them, then an RMS norm of o (per head, or over the concatenated heads; with or without a
+// weight) and an output gate silu(g) or sigmoid(g). Key and value sizes may differ. Three launches:
+//   prep   (token, head) parallel: the fp32 per-channel triples {a, k_scale k, q_scale q} and the values.
 //   scan   the recurrence. Column v of S depends on no other column, so a head's value columns are split
 //          into slices of 8 NC and every (sequence, head, slice) is one wave: lane = (key group of eight,
 //          columns c + 8 n for n < NC), ceil(D / 8) x NC state entries in registers; per token one FMA pair
@@ -43,11 +45,24 @@ __global__ __launch_bounds__(256) void linear_prep_kernel(LinearAttnArgs p, floa
   if (t >= p.query_start[p.S]) return;  // padding rows of a graph bucket
   const int HD = p.H * p.D, HV = p.H * p.V;
   const float inv_tau = 1.f / p.tau;
+  const float pos = p.rot_dims > 0 ? (float)p.positions[t] : 0.f;
+  const int half = p.rot_dims >> 1;
   for (int e = threadIdx.x; e < HD; e += blockDim.x) {
     float q = ldx(p.q, (int64_t)t * p.ldq + e, p.f32), k = ldx(p.k, (int64_t)t * p.ldk + e, p.f32);
     if (p.in_silu) { q = silu_f(q); k = silu_f(k); }
+    const int d = e % p.D;
+    if (d < p.rot_dims) {  // the pair's other entry, then (u, v) -> (u c - v s, v c + u s)
+      const bool first = p.rot_half ? d < half : !(d & 1);
+      const int eo = p.rot_half ? (first ? e + half : e - half) : (e ^ 1);
+      float qo = ldx(p.q, (int64_t)t * p.ldq + eo, p.f32), ko = ldx(p.k, (int64_t)t * p.ldk + eo, p.f32);
+      if (p.in_silu) { qo = silu_f(qo); ko = silu_f(ko); }
+      const float ang = pos * p.inv_freq[p.rot_half ? (first ? d : d - half) : (d >> 1)];
+      const float cs = cosf(ang), sn = sinf(ang);
+      q = first ? q * cs - qo * sn : q * cs + qo * sn;
+      k = first ? k * cs - ko * sn : k * cs + ko * sn;
+    }
     const float a = p.z != nullptr ? expf(log_sigmoid(p.z[(int64_t)t * p.ldz + e]) * inv_tau) : p.head_decay[e / p.D];
-    vec[(int64_t)t * HD + e] = make_float4(a, k, q * p.q_scale, 0.f);
+    vec[(int64_t)t * HD + e] = make_float4(a, k * p.k_scale, q * p.q_scale, 0.f);
   }
   for (int e = threadIdx.x; e < HV; e += blockDim.x) {
     const float v = ldx(p.v, (int64_t)t * p.ldv + e, p.f32);
@@ -255,7 +270,7 @@ __global__ __launch_bounds__(256) void linear_finish_kernel(LinearAttnArgs p, co
     for (int e = threadIdx.x; e < HV; e += blockDim.x) ss = fmaf(o[e], o[e], ss);
     ss = block_reduce_sum(ss, red);
     const float inv = 1.f / sqrtf(ss / (float)HV + p.eps);
-    for (int e = threadIdx.x; e < HV; e += blockDim.x) emit(e, o[e] * inv * p.nw[e]);
+    for (int e = threadIdx.x; e < HV; e += blockDim.x) emit(e, o[e] * inv * (p.nw != nullptr ? p.nw[e] : 1.f));
     return;
   }
   const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -264,7 +279,7 @@ __global__ __launch_bounds__(256) void linear_finish_kernel(LinearAttnArgs p, co
     for (int c = lane; c < V; c += 64) ss = fmaf(o[h * V + c], o[h * V + c], ss);
     ss = wave_reduce_sum(ss);
     const float inv = 1.f / sqrtf(ss / (float)V + p.eps);
-    for (int c = lane; c < V; c += 64) emit(h * V + c, o[h * V + c] * inv * p.nw[c]);
+    for (int c = lane; c < V; c += 64) emit(h * V + c, o[h * V + c] * inv * (p.nw != nullptr ? p.nw[c] : 1.f));
   }
 }
 

@@ -1,8 +1,9 @@
 // Row-wise kernels of layered hybrid models over an fp32 residual stream: embedding gather into
 // fp32, RMS norm with a scalar or vector weight (fp32 statistics, bf16 or fp32 rows in and out,
-// optional row gather), the gated residual update of a parallel layer, and mixture-of-experts
-// routing (sigmoid scores with a selection-only correction, top-k, counting sort by expert, weighted
-// combine). Every kernel reads its sizes from arguments and its per-step metadata from device
+// optional row gather), a tanh norm without statistics, the gated residual update of a parallel layer,
+// the read / write of a sublayer over several learned-weight copies of the stream, and mixture-of-experts
+// routing (sigmoid or softmax scores with an optional selection-only correction, top-k, counting sort by
+// expert, weighted combine with an optional shared-expert row). Every kernel reads its sizes from arguments and its per-step metadata from device
 // memory, so the launches are graph-capturable.
 #include "common.h"
 #include "seq_launchers.h"
@@ -127,13 +128,74 @@ __global__ __launch_bounds__(256) void post_norm_add_kernel(PostNormArgs a) {
   }
 }
 
+__global__ __launch_bounds__(256) void tanh_norm_rows_kernel(const float* __restrict__ x, int64_t ldx_,
+                                                              const int32_t* __restrict__ rows,
+                                                              const float* __restrict__ alpha, const float* __restrict__ w,
+                                                              const float* __restrict__ b, void* __restrict__ y,
+                                                              int64_t ldy, int y_f32, int n) {
+  const int m = blockIdx.x;
+  const int64_t src = rows ? rows[m] : m;
+  const float al = alpha[0];
+  for (int c = threadIdx.x; c < n; c += blockDim.x)
+    stx(y, (int64_t)m * ldy + c, y_f32, fmaf(tanhf(al * x[src * ldx_ + c]), w[c], b[c]));
+}
+
+// one thread per (token, column): the S copies of the element are read, mixed and written by the same thread
+__global__ __launch_bounds__(256) void hyper_mix_kernel(HyperArgs a) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (int64_t)a.T * a.W) return;
+  const int c = (int)(i % a.W);
+  const int S = a.S;
+  float x[kMaxStreams];
+#pragma unroll
+  for (int s = 0; s < kMaxStreams; ++s) x[s] = s < S ? a.xs[s * a.plane + i] : 0.f;
+  if (a.y != nullptr) {
+    const float yv = ldx(a.y, i, a.y_f32);
+    float nx[kMaxStreams];
+#pragma unroll
+    for (int t = 0; t < kMaxStreams; ++t) {
+      float v = 0.f;
+      if (t < S) {
+#pragma unroll
+        for (int s = 0; s < kMaxStreams; ++s)
+          if (s < S) v = fmaf(a.mix[s * S + t], x[s], v);
+        v = fmaf(a.out_w[t], yv, v);
+        a.xs[t * a.plane + i] = v;
+      }
+      nx[t] = v;
+    }
+#pragma unroll
+    for (int s = 0; s < kMaxStreams; ++s) x[s] = nx[s];
+  }
+  if (a.read_w != nullptr) {
+    float u = 0.f;
+#pragma unroll
+    for (int s = 0; s < kMaxStreams; ++s)
+      if (s < S) u = fmaf(a.read_w[s], x[s], u);
+    stx(a.h_out, i, a.h_f32, fmaf(tanhf(a.alpha[0] * u), a.w[c], a.b[c]));
+  }
+  if (a.sum_out != nullptr) {
+    float u = 0.f;
+#pragma unroll
+    for (int s = 0; s < kMaxStreams; ++s)
+      if (s < S) u += x[s];
+    a.sum_out[i] = u;
+  }
+}
+
 // one thread per token: `top` rounds of arg-max over the corrected scores (lowest index wins a tie)
 __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ z, const float* __restrict__ corr,
-                                                        int T, int E, int top, float norm_eps,
+                                                        int T, int E, int top, float norm_eps, int softmax, float scale,
                                                         int32_t* __restrict__ idx, float* __restrict__ wts) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= T) return;
   const float* zr = z + (int64_t)t * E;
+  float zmax = -INFINITY, den = 1.f;
+  if (softmax) {  // scores over all experts: exp(z - max) / sum
+    for (int e = 0; e < E; ++e) zmax = fmaxf(zmax, zr[e]);
+    den = 0.f;
+    for (int e = 0; e < E; ++e) den += expf(zr[e] - zmax);
+  }
   float sum = 0.f;
   for (int c = 0; c < top; ++c) {
     int best = -1;
@@ -142,7 +204,7 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
       bool taken = false;
       for (int d = 0; d < c; ++d) taken |= idx[(int64_t)t * top + d] == e;
       if (taken) continue;
-      const float s = sigm(zr[e]);
+      const float s = softmax ? expf(zr[e] - zmax) / den : sigm(zr[e]);
       const float v = s + (corr ? corr[e] : 0.f);
       if (best < 0 || v > bv) { best = e; bv = v; bs = s; }
     }
@@ -151,7 +213,7 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
     sum += bs;
   }
   const float inv = 1.f / (sum + norm_eps);
-  for (int c = 0; c < top; ++c) wts[(int64_t)t * top + c] *= inv;
+  for (int c = 0; c < top; ++c) wts[(int64_t)t * top + c] = wts[(int64_t)t * top + c] * inv * scale;
 }
 
 // single workgroup: histogram, exclusive scan, placement (token order inside a group is arbitrary:
@@ -182,14 +244,16 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const int32_t* __restric
 }
 
 __global__ __launch_bounds__(256) void moe_combine_kernel(const void* __restrict__ y, const int32_t* __restrict__ pos,
-                                                           const float* __restrict__ wts, int W, int top, int f32,
-                                                           void* __restrict__ out) {
+                                                           const float* __restrict__ wts, int W, int top, int y_f32,
+                                                           const void* __restrict__ add, void* __restrict__ out,
+                                                           int out_f32) {
   const int t = blockIdx.x;
   for (int c = threadIdx.x; c < W; c += blockDim.x) {
     float a = 0.f;
     for (int k = 0; k < top; ++k)
-      a = fmaf(wts[(int64_t)t * top + k], ldx(y, (int64_t)pos[(int64_t)t * top + k] * W + c, f32), a);
-    stx(out, (int64_t)t * W + c, f32, a);
+      a = fmaf(wts[(int64_t)t * top + k], ldx(y, (int64_t)pos[(int64_t)t * top + k] * W + c, y_f32), a);
+    if (add != nullptr) a += ldx(add, (int64_t)t * W + c, out_f32);
+    stx(out, (int64_t)t * W + c, out_f32, a);
   }
 }
 
@@ -233,10 +297,23 @@ void launch_gated_residual(float* x, const void* y1, const void* g1, int64_t ldg
   hipLaunchKernelGGL(gated_residual_kernel, dim3(T), dim3(256), 0, st, x, y1, g1, ldg1, b1, y2, g2, ldg2, b2, f32, W);
 }
 
-void launch_moe_route(const float* z, const float* corr, int T, int E, int top, float norm_eps, int32_t* idx,
-                      float* wts, hipStream_t st) {
+void launch_moe_route(const float* z, const float* corr, int T, int E, int top, float norm_eps, int softmax, float scale,
+                      int32_t* idx, float* wts, hipStream_t st) {
   if (T <= 0) return;
-  hipLaunchKernelGGL(moe_route_kernel, dim3((T + 63) / 64), dim3(64), 0, st, z, corr, T, E, top, norm_eps, idx, wts);
+  hipLaunchKernelGGL(moe_route_kernel, dim3((T + 63) / 64), dim3(64), 0, st, z, corr, T, E, top, norm_eps, softmax, scale,
+                     idx, wts);
+}
+
+void launch_tanh_norm_rows(const float* x, int64_t ldx_, const int32_t* rows, const float* alpha, const float* w,
+                           const float* b, void* y, int64_t ldy, int y_f32, int M, int n, hipStream_t st) {
+  if (M <= 0) return;
+  hipLaunchKernelGGL(tanh_norm_rows_kernel, dim3(M), dim3(256), 0, st, x, ldx_, rows, alpha, w, b, y, ldy, y_f32, n);
+}
+
+void launch_hyper_mix(const HyperArgs& a, hipStream_t st) {
+  const int64_t tot = (int64_t)a.T * a.W;
+  if (tot <= 0 || a.S <= 0) return;
+  hipLaunchKernelGGL(hyper_mix_kernel, dim3((unsigned)((tot + 255) / 256)), dim3(256), 0, st, a);
 }
 
 void launch_moe_sort(const int32_t* idx, int T, int E, int top, int32_t* rows, int32_t* pos, int32_t* off,
@@ -246,10 +323,10 @@ void launch_moe_sort(const int32_t* idx, int T, int E, int top, int32_t* rows, i
                      pos, off);
 }
 
-void launch_moe_combine(const void* y, const int32_t* pos, const float* wts, int T, int W, int top, int f32,
-                        void* out, hipStream_t st) {
+void launch_moe_combine(const void* y, const int32_t* pos, const float* wts, int T, int W, int top, int y_f32,
+                        const void* add, void* out, int out_f32, hipStream_t st) {
   if (T <= 0) return;
-  hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(256), 0, st, y, pos, wts, W, top, f32, out);
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(256), 0, st, y, pos, wts, W, top, y_f32, add, out, out_f32);
 }
 
 }  // namespace vgate

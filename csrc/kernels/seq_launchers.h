@@ -105,6 +105,11 @@ struct WindowArgs {
   const float* inv_freq = nullptr;      // [rot_dims / 2]
   const float* v_freq = nullptr;        // [V / 2]: values are turned by their position (null: not)
   const float* sink = nullptr;          // [H] logits that only enter the softmax denominator (null: none)
+  // distance term of a token's score, n = query position - key position (0: none; not with pooled blocks):
+  // 1: -bias_a[h] * ln(1 + bias_b[h] * n); 2: bias_a[h][min(n, bias_n - 1)]
+  int bias_kind = 0, bias_n = 0, bias_lds = 0;   // bias_lds: the MFMA kernels stage a workgroup's heads' table in LDS
+  const float* bias_a = nullptr; const float* bias_b = nullptr;
+  const void* gate = nullptr; int64_t ldg = 0;   // [T][H * V] rows (activation dtype): out *= sigmoid(gate); null: none
   const int32_t* positions = nullptr;   // [T]
   const int32_t* slots = nullptr;       // [T] page * tokens-per-page + offset of each token (-1: padding)
   const int32_t* block_tables = nullptr; const int32_t* context_lens = nullptr; const int32_t* query_start = nullptr;
@@ -114,10 +119,11 @@ struct WindowArgs {
 size_t window_attn_lds_bytes(const WindowArgs& a, int heads_per_block);
 bool window_attn_fits(const WindowArgs& a);   // sizes the kernels' LDS and register budgets take
 // q / k norm (qw, kw null: none; norm_all: one norm over the whole projection) + rotation + paged stores; q_out [T][H * D];
+// the query of head h at position p is multiplied by q_head_scale[h] (null: 1) * (1 + q_temp_coef ln(floor((p + 1) / q_temp_every) + 1));
 // vt: optional second, transposed bf16 copy of the values [pages][G][V][page]
 void launch_window_write(const WindowArgs& a, const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v,
                          int64_t ldv, const float* qw, const float* kw, float eps, int norm_all, void* q_out, void* vt,
-                         hipStream_t st);
+                         const float* q_head_scale, float q_temp_coef, int q_temp_every, hipStream_t st);
 // pooled rows of the blocks this step's tokens complete
 void launch_window_pool(const WindowArgs& a, hipStream_t st);
 // out[t][h][:V] = softmax over (pooled blocks before the window, window tokens [, sink]) of scale q . key, times values
@@ -132,9 +138,14 @@ struct LinearAttnArgs {
   int64_t ldq = 0, ldk = 0, ldv = 0, ldg = 0;   // activation dtype rows: q, k [H * D]; v, g [H * V]
   const float* z = nullptr; int64_t ldz = 0;    // decay logits per key channel (null: head_decay)
   const float* head_decay = nullptr;            // [H]
-  float tau = 1.f, q_scale = 1.f, eps = 0.f;
+  float tau = 1.f, q_scale = 1.f, k_scale = 1.f, eps = 0.f;
   int in_silu = 0, norm_all = 0, gate_silu = 0;
-  const float* nw = nullptr;                    // [V], or [H * V] with norm_all
+  // rotary positions on the leading rot_dims (even) entries of every q / k head: rot_half pairs entry i with
+  // i + rot_dims / 2, otherwise 2i with 2i + 1; angle = positions[t] * inv_freq[pair]
+  int rot_dims = 0, rot_half = 1;
+  const float* inv_freq = nullptr;              // [rot_dims / 2]
+  const int32_t* positions = nullptr;           // [T] (read when rot_dims > 0)
+  const float* nw = nullptr;                    // [V], or [H * V] with norm_all; null: no weight
   float* state = nullptr;                       // [slots][H][D][V]
   const int32_t* state_slots = nullptr; const int32_t* context_lens = nullptr; const int32_t* query_start = nullptr;
   void* out = nullptr; int64_t ldo = 0;
@@ -149,15 +160,37 @@ size_t linear_attn_scratch_floats(int T, int S, int H, int D, int V);
 // T rows; scratch: linear_attn_scratch_floats() floats, 16-B aligned
 void launch_linear_attn(const LinearAttnArgs& a, int T, float* scratch, hipStream_t st);
 
-// idx, wts [T][top]: the `top` largest of sigmoid(z) + corr; wts = sigmoid(z) of the chosen / their sum
-void launch_moe_route(const float* z, const float* corr, int T, int E, int top, float norm_eps, int32_t* idx,
-                      float* wts, hipStream_t st);
+// idx, wts [T][top]: the `top` largest of s + corr with s = sigmoid(z) or, with `softmax`, softmax(z) over all E;
+// wts = s of the chosen / (their sum + norm_eps) * scale
+void launch_moe_route(const float* z, const float* corr, int T, int E, int top, float norm_eps, int softmax, float scale,
+                      int32_t* idx, float* wts, hipStream_t st);
 // counting sort of the T * top (token, choice) pairs by expert: rows[p] = token, pos[t * top + c] = p,
 // off[E + 1] = group boundaries
 void launch_moe_sort(const int32_t* idx, int T, int E, int top, int32_t* rows, int32_t* pos, int32_t* off,
                      hipStream_t st);
-// out[t] = sum_c wts[t][c] * y[pos[t][c]]
-void launch_moe_combine(const void* y, const int32_t* pos, const float* wts, int T, int W, int top, int f32,
-                        void* out, hipStream_t st);
+// out[t] = sum_c wts[t][c] * y[pos[t][c]] [+ add[t]] (add: out's dtype)
+void launch_moe_combine(const void* y, const int32_t* pos, const float* wts, int T, int W, int top, int y_f32,
+                        const void* add, void* out, int out_f32, hipStream_t st);
+
+// y[m][:] = tanh(alpha[0] * x[row(m)][:]) * w + b   (x fp32; a norm without statistics)
+void launch_tanh_norm_rows(const float* x, int64_t ldx, const int32_t* rows, const float* alpha, const float* w,
+                           const float* b, void* y, int64_t ldy, int y_f32, int M, int n, hipStream_t st);
+
+// Several fp32 copies of the residual stream, xs [S][T][W] (plane stride `plane`), that a sublayer reads through
+// learned weights and writes back to. One launch does a sublayer's write and the next one's read:
+//   y given:      xs[t] <- sum_s mix[s][t] xs[s] + out_w[t] * y      (all copies at once from the old ones)
+//   read_w given: h_out = tanh(alpha[0] * sum_s read_w[s] xs[s]) * w + b   (from the new copies)
+//   sum_out given: the sum of the new copies
+constexpr int kMaxStreams = 8;
+struct HyperArgs {
+  float* xs = nullptr; int64_t plane = 0;
+  const void* y = nullptr; int y_f32 = 0;
+  const float* mix = nullptr; const float* out_w = nullptr;
+  const float* read_w = nullptr; const float* alpha = nullptr; const float* w = nullptr; const float* b = nullptr;
+  void* h_out = nullptr; int h_f32 = 0;
+  float* sum_out = nullptr;
+  int S = 0, T = 0, W = 0;
+};
+void launch_hyper_mix(const HyperArgs& a, hipStream_t st);
 
 }  // namespace vgate

@@ -30,6 +30,10 @@
 //                             tiles the eight values are gathered from the pooled rows.
 //               Window, causal and pooled-block visibility are per-row masks on whole tiles, and tiles sit
 //               at fixed absolute key positions, so a row's sums do not depend on which rows share its wave.
+// Distance term (no pooled blocks then): a score may carry a bias that depends on the head and the distance
+//               n = i - j alone, -r1[h] ln(1 + r2[h] n) or a table entry tab[h][min(n, last)]; the MFMA kernels
+//               compute it in log2 units beside the mask (the table of a workgroup's heads staged in LDS when
+//               it fits). An output gate multiplies the normalised result by sigmoid(gate) in the epilogue.
 // Every row of every kernel depends only on its own sequence's cache rows, in an order fixed by the
 // position, so results do not depend on how a prompt is cut or what else is in the batch.
 #include "common.h"
@@ -60,7 +64,8 @@ __global__ __launch_bounds__(256) void window_write_kernel(WindowArgs a, const v
                                                             const void* __restrict__ v, int64_t ldv,
                                                             const float* __restrict__ qw, const float* __restrict__ kw,
                                                             float eps, int norm_all, void* __restrict__ q_out,
-                                                            bf16_t* __restrict__ vt) {
+                                                            bf16_t* __restrict__ vt, const float* __restrict__ q_head_scale,
+                                                            float q_temp_coef, int q_temp_every) {
   extern __shared__ float lds[];
   const int H = a.H, G = a.G, D = a.D, V = a.V;
   float* xs = lds;                    // [(H + G) * D] q heads then k heads
@@ -94,6 +99,8 @@ __global__ __launch_bounds__(256) void window_write_kernel(WindowArgs a, const v
     __syncthreads();
   }
   const float pos = (float)a.positions[t];
+  // query temperature of the position: 1 + coef ln(floor((p + 1) / every) + 1)
+  const float qgrow = q_temp_coef != 0.f ? 1.f + q_temp_coef * logf((float)((a.positions[t] + 1) / q_temp_every) + 1.f) : 1.f;
   const int page = a.page;
   const int64_t pg = slot / page, off = slot % page;
   for (int e = tid; e < (H + G) * D; e += 256) {
@@ -112,7 +119,7 @@ __global__ __launch_bounds__(256) void window_write_kernel(WindowArgs a, const v
     } else {
       o = xs[h * D + i] * sc * (w ? w[wo + i] : 1.f);
     }
-    if (isq) stx(q_out, (int64_t)t * H * D + e, a.f32, o);
+    if (isq) stx(q_out, (int64_t)t * H * D + e, a.f32, o * (q_head_scale != nullptr ? q_head_scale[h] * qgrow : qgrow));
     else stx(a.kc, ((pg * G + (h - H)) * page + off) * D + i, a.f32, o);
   }
   const int vrot = a.v_freq != nullptr ? 2 * (V / 2) : 0;
@@ -261,7 +268,13 @@ __global__ __launch_bounds__(256) void window_attn_kernel(WindowArgs a, const vo
         for (int c = c0; c < c1; ++c) d = fmaf(qp[c], kp[c], d);
       }
       d += __shfl_xor(d, 1, 64);
-      if (on && half == 0) sc[h * KT + jj] = (j0 + jj < nkeys) ? d * scale : -INFINITY;
+      float bias = 0.f;
+      if (a.bias_kind != 0 && on && j0 + jj >= nb && j0 + jj < nkeys) {  // (token keys: kj - nb keys after lo)
+        const int n = pos - (lo + j0 + jj - nb);
+        bias = a.bias_kind == 1 ? -a.bias_a[h0 + h] * logf(1.f + a.bias_b[h0 + h] * (float)n)
+                                : a.bias_a[(int64_t)(h0 + h) * a.bias_n + min(n, a.bias_n - 1)];
+      }
+      if (on && half == 0) sc[h * KT + jj] = (j0 + jj < nkeys) ? d * scale + bias : -INFINITY;
     }
     __syncthreads();
     if (tid < nh) {
@@ -269,13 +282,13 @@ __global__ __launch_bounds__(256) void window_attn_kernel(WindowArgs a, const vo
       float m1 = m0;
       for (int jj = 0; jj < KT; ++jj) m1 = fmaxf(m1, sc[tid * KT + jj]);
       const float al = expf(m0 - m1);  // m0 = -inf on the first tile: 0
-      float l = lrun[tid] * al;
+      float l = 0.f;  // the tile's own sum first: the running sum takes one rounding per tile, not per key
       for (int jj = 0; jj < KT; ++jj) {
         const float pj = expf(sc[tid * KT + jj] - m1);
         sc[tid * KT + jj] = pj;
         l += pj;
       }
-      mrun[tid] = m1; lrun[tid] = l; alpha[tid] = al;
+      mrun[tid] = m1; lrun[tid] = fmaf(lrun[tid], al, l); alpha[tid] = al;
     }
     __syncthreads();
 #pragma unroll
@@ -283,20 +296,23 @@ __global__ __launch_bounds__(256) void window_attn_kernel(WindowArgs a, const vo
       const int o = tid + i * 256;
       if (o < nh * V) {
         const int h = o / V, c = o % V;
-        float x = acc[i] * alpha[h];
+        float x = 0.f;
         const float* pp = sc + h * KT;
 #pragma unroll
         for (int jj = 0; jj < KT; ++jj) x = fmaf(pp[jj], vs[jj * VP + c], x);
-        acc[i] = x;
+        acc[i] = fmaf(acc[i], alpha[h], x);
       }
     }
   }
   __syncthreads();
+  auto gated = [&](int o, float y) {  // o: (head - h0) * V + column
+    return a.gate != nullptr ? y / (1.f + expf(-ldx(a.gate, (int64_t)t * a.ldg + (int64_t)h0 * V + o, a.f32))) : y;
+  };
   if (a.v_freq == nullptr) {
 #pragma unroll
     for (int i = 0; i < MAXACC; ++i) {
       const int o = tid + i * 256;
-      if (o < nh * V) stx(out, ((int64_t)t * a.H + h0) * V + o, a.f32, acc[i] / lrun[o / V]);
+      if (o < nh * V) stx(out, ((int64_t)t * a.H + h0) * V + o, a.f32, gated(o, acc[i] / lrun[o / V]));
     }
     return;
   }
@@ -317,7 +333,7 @@ __global__ __launch_bounds__(256) void window_attn_kernel(WindowArgs a, const vo
       const float cs = cosf(ang), sn = sinf(ang);
       y = (i & 1) ? (x1 * cs + x0 * sn) : (x0 * cs - x1 * sn);
     }
-    stx(out, ((int64_t)t * a.H + h0) * V + o, a.f32, y);
+    stx(out, ((int64_t)t * a.H + h0) * V + o, a.f32, gated(o, y));
   }
 }
 
@@ -358,16 +374,39 @@ __device__ __forceinline__ float group16_sum(float v) {
   return v;
 }
 
+// Distance term of the MFMA kernels, in log2 units. Per C-layout row of a lane: bw / bx are (r1, r2) of the
+// row's head for the logarithmic penalty; bo is the row's offset into the table of the workgroup's heads.
+constexpr float LOG2E = 1.4426950408889634f;
+__device__ __forceinline__ void bias_stage(const WindowArgs& a, float* btab, int g, int rep, int tid, int nthreads) {
+  if (a.bias_kind == 2 && a.bias_lds)
+    for (int e = tid; e < rep * a.bias_n; e += nthreads) btab[e] = a.bias_a[(int64_t)g * rep * a.bias_n + e] * LOG2E;
+}
+__device__ __forceinline__ void bias_row(const WindowArgs& a, int g, int rep, int r, bool ok, float& bw, float& bx, int& bo) {
+  const int hr = ok ? r % rep : 0;
+  bw = bx = 0.f;
+  bo = hr * a.bias_n;
+  if (a.bias_kind == 1) { bw = a.bias_a[g * rep + hr]; bx = a.bias_b[g * rep + hr]; }
+}
+__device__ __forceinline__ float bias_of(const WindowArgs& a, const float* btab, int g, int rep, float bw, float bx, int bo,
+                                         int n) {
+  n = max(n, 0);  // (a key the row does not see: masked by the caller)
+  if (a.bias_kind == 1) return -bw * __log2f(fmaf(bx, (float)n, 1.f));
+  const int idx = bo + min(n, a.bias_n - 1);
+  return a.bias_lds ? btab[idx] : a.bias_a[(int64_t)g * rep * a.bias_n + idx] * LOG2E;
+}
+__device__ __forceinline__ float gate_of(const bf16_t* grow, int col) { return 1.f / (1.f + __expf(-bf2f(grow[col]))); }
+
 // NCT: 16-column tiles of the value (V <= 16 NCT); NQF: 32-wide fragments of a query row (D <= 32 NQF).
 // D % 8 == 0 (host-checked): every key fragment is one unconditional 16-B load; a fragment past the row's
 // end or the value's last column is read from a clamped address: its partner (zero Q fragment) or its
 // output column (never stored) makes the value irrelevant, and cached values are always finite.
 constexpr int LG = 4;
 // NW: waves of a workgroup, which share out the key tiles of its 16 rows
-template <int NCT, int NQF, int NW>
+template <int NCT, int NQF, int NW, int BIAS>
 __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a, const bf16_t* __restrict__ q,
                                                                 float scale_log2e, const bf16_t* __restrict__ vt,
                                                                 int num_pages, bf16_t* __restrict__ out) {
+  extern __shared__ float btab[];  // BIAS: the distance table of this workgroup's heads (when it is staged)
   __shared__ __attribute__((aligned(16))) bf16_t pl[NW][16][40];
   __shared__ float mrg_m[NW][16], mrg_l[NW][16];
   __shared__ float mrg_o[16][16 * NCT];  // the merged weighted values of the 16 rows
@@ -387,6 +426,10 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
   // (max, sum, weighted values) through LDS: four times the waves to hide the cache's latency behind
   const int row0 = tile * 16;
   if (row0 >= nrows) return;  // (workgroup-uniform)
+  if (BIAS) {
+    bias_stage(a, btab, g, rep, threadIdx.x, 64 * NW);
+    __syncthreads();
+  }
   const bf16_t* kc = reinterpret_cast<const bf16_t*>(a.kc);
   const bf16_t* kp = reinterpret_cast<const bf16_t*>(a.kp);
   const bf16_t* vp = reinterpret_cast<const bf16_t*>(a.vp);
@@ -402,6 +445,8 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
   // C-layout rows of this lane: row0 + 4 lg + i; what each sees: tokens [lo, hi], pooled blocks [0, nbv)
   int hi[4], lo[4], nbv[4];
   float m[4], lsum[4];
+  float bw[BIAS ? 4 : 1], bx[BIAS ? 4 : 1];
+  int bo[BIAS ? 4 : 1];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r = row0 + 4 * lg + i;
@@ -410,6 +455,7 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
     hi[i] = ok ? p : -1;
     lo[i] = p - a.window + 1;
     nbv[i] = (ok && P > 0) ? max(0, lo[i]) / P : 0;
+    if (BIAS) bias_row(a, g, rep, r, ok, bw[i], bx[i], bo[i]);
     const bool sk = ok && a.sink != nullptr && wv == 0;  // the sink counts once
     m[i] = sk ? a.sink[g * rep + r % rep] * 1.4426950408889634f : -INFINITY;
     lsum[i] = (sk && lr == 0) ? 1.f : 0.f;
@@ -469,8 +515,12 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
     for (int i = 0; i < 4; ++i) {
       const bool vis0 = pooled ? c0 < nbv[i] : (c0 >= lo[i] && c0 <= hi[i]);
       const bool vis1 = pooled ? c1 < nbv[i] : (c1 >= lo[i] && c1 <= hi[i]);
-      const float v0 = vis0 ? s0[i] * scale_log2e : -INFINITY;
-      const float v1 = vis1 ? s1[i] * scale_log2e : -INFINITY;
+      float v0 = vis0 ? s0[i] * scale_log2e : -INFINITY;
+      float v1 = vis1 ? s1[i] * scale_log2e : -INFINITY;
+      if (BIAS) {  // (never with pooled tiles)
+        if (vis0) v0 += bias_of(a, btab, g, rep, bw[i], bx[i], bo[i], hi[i] - c0);
+        if (vis1) v1 += bias_of(a, btab, g, rep, bw[i], bx[i], bo[i], hi[i] - c1);
+      }
       const float mnew = fmaxf(m[i], group16_max(fmaxf(v0, v1)));
       const float ms = (mnew == -INFINITY) ? 0.f : mnew;  // a row that has seen no key yet
       al[i] = exp2f(m[i] - ms);
@@ -571,6 +621,8 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
     const bool ok = r < nrows;
     const float fp = -(float)(pos0 + (ok ? r / rep : 0));
     bf16_t* orow = out + ((int64_t)(t0 + (ok ? r / rep : 0)) * H + g * rep + (ok ? r % rep : 0)) * V;
+    const bf16_t* grow = a.gate == nullptr ? nullptr : reinterpret_cast<const bf16_t*>(a.gate) +
+        (int64_t)(t0 + (ok ? r / rep : 0)) * a.ldg + (int64_t)(g * rep + (ok ? r % rep : 0)) * V;
 #pragma unroll
     for (int ct = 0; ct < NCT; ++ct) {
       if (SHARE && ct % NW != wv) continue;  // wave-uniform
@@ -584,7 +636,7 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
           y = (col & 1) ? (y * cs + other * sn) : (y * cs - other * sn);
         }
       }
-      if (ok && ct < nct && col < V) orow[col] = f2bf(y);
+      if (ok && ct < nct && col < V) orow[col] = f2bf(grow != nullptr ? y * gate_of(grow, col) : y);
     }
   }
 }
@@ -593,10 +645,11 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
 // and transposed values are brought into LDS once per workgroup (two buffers: tile t + 1 is asked for before
 // tile t is computed, written after it, one barrier per tile), and every wave takes its fragments from there.
 // Pooled tiles come first and are read straight from the pooled caches by each wave, as in the kernel above.
-template <int NCT, int NQF>
+template <int NCT, int NQF, int BIAS>
 __global__ __launch_bounds__(256) void window_attn_tiled_kernel(WindowArgs a, const bf16_t* __restrict__ q,
                                                                  float scale_log2e, const bf16_t* __restrict__ vt,
                                                                  int num_pages, bf16_t* __restrict__ out) {
+  extern __shared__ float btab[];  // BIAS: the distance table of this workgroup's heads (when it is staged)
   constexpr int DP = 32 * NQF + 8;  // padded row of a staged key (bf16): rows 16 B apart in the banks
   constexpr int VP = 40;            // padded row of a staged value column: 32 keys + 8
   constexpr int NKC = (32 * 4 * NQF + 255) / 256, NVC = (4 * 16 * NCT + 255) / 256;  // 16-B pieces per thread
@@ -625,6 +678,7 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(WindowArgs a, co
   const int nqf = (D + 31) >> 5, nct = (V + 15) >> 4, d8 = D >> 3;
   for (int e = tid; e < 2 * 32 * DP / 8; e += 256) reinterpret_cast<uint4*>(&kl[0][0][0])[e] = make_uint4(0, 0, 0, 0);
   for (int e = tid; e < 2 * 16 * NCT * VP / 8; e += 256) reinterpret_cast<uint4*>(&vl[0][0][0])[e] = make_uint4(0, 0, 0, 0);
+  if (BIAS) bias_stage(a, btab, g, rep, tid, 256);  // (the barrier before the first tile covers it)
   bf16x8 qf[NQF];
   {
     const int r = row0 + lr;
@@ -635,6 +689,8 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(WindowArgs a, co
   }
   int hi[4], lo[4], nbv[4];
   float m[4], lsum[4];
+  float bw[BIAS ? 4 : 1], bx[BIAS ? 4 : 1];
+  int bo[BIAS ? 4 : 1];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r = row0 + 4 * lg + i;
@@ -643,6 +699,7 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(WindowArgs a, co
     hi[i] = ok ? p : -1;
     lo[i] = p - a.window + 1;
     nbv[i] = (ok && P > 0) ? max(0, lo[i]) / P : 0;
+    if (BIAS) bias_row(a, g, rep, r, ok, bw[i], bx[i], bo[i]);
     const bool sk = ok && a.sink != nullptr;
     m[i] = sk ? a.sink[g * rep + r % rep] * 1.4426950408889634f : -INFINITY;
     lsum[i] = (sk && lr == 0) ? 1.f : 0.f;
@@ -669,8 +726,12 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(WindowArgs a, co
     for (int i = 0; i < 4; ++i) {
       const bool vis0 = pooled ? c0 < nbv[i] : (c0 >= lo[i] && c0 <= hi[i]);
       const bool vis1 = pooled ? c1 < nbv[i] : (c1 >= lo[i] && c1 <= hi[i]);
-      const float v0 = vis0 ? s0[i] * scale_log2e : -INFINITY;
-      const float v1 = vis1 ? s1[i] * scale_log2e : -INFINITY;
+      float v0 = vis0 ? s0[i] * scale_log2e : -INFINITY;
+      float v1 = vis1 ? s1[i] * scale_log2e : -INFINITY;
+      if (BIAS) {  // (never with pooled tiles)
+        if (vis0) v0 += bias_of(a, btab, g, rep, bw[i], bx[i], bo[i], hi[i] - c0);
+        if (vis1) v1 += bias_of(a, btab, g, rep, bw[i], bx[i], bo[i], hi[i] - c1);
+      }
       const float mnew = fmaxf(m[i], group16_max(fmaxf(v0, v1)));
       const float ms = (mnew == -INFINITY) ? 0.f : mnew;
       al[i] = exp2f(m[i] - ms);
@@ -797,6 +858,8 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(WindowArgs a, co
     const bool ok = r < nrows;
     const float fp = -(float)(pos0 + (ok ? r / rep : 0));
     bf16_t* orow = out + ((int64_t)(t0 + (ok ? r / rep : 0)) * H + g * rep + (ok ? r % rep : 0)) * V;
+    const bf16_t* grow = a.gate == nullptr ? nullptr : reinterpret_cast<const bf16_t*>(a.gate) +
+        (int64_t)(t0 + (ok ? r / rep : 0)) * a.ldg + (int64_t)(g * rep + (ok ? r % rep : 0)) * V;
 #pragma unroll
     for (int ct = 0; ct < NCT; ++ct) {
       const int col = 16 * ct + lr;
@@ -809,15 +872,16 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(WindowArgs a, co
           y = (col & 1) ? (y * cs + other * sn) : (y * cs - other * sn);
         }
       }
-      if (ok && ct < nct && col < V) orow[col] = f2bf(y);
+      if (ok && ct < nct && col < V) orow[col] = f2bf(grow != nullptr ? y * gate_of(grow, col) : y);
     }
   }
 }
 
-template <int NCT, int NQF>
+template <int NCT, int NQF, int BIAS>
 void launch_window_mfma(const WindowArgs& a, const void* q, float scale, const void* vt, int num_pages, void* out,
                         hipStream_t st) {
   const int rep = a.H / a.G;
+  const size_t dyn = (BIAS && a.bias_kind == 2 && a.bias_lds) ? (size_t)rep * a.bias_n * sizeof(float) : 0;
   const int blocks = (a.T * rep + 15) / 16 + a.S;
   const bf16_t* qp = reinterpret_cast<const bf16_t*>(q);
   const bf16_t* vp = reinterpret_cast<const bf16_t*>(vt);
@@ -827,12 +891,20 @@ void launch_window_mfma(const WindowArgs& a, const void* q, float scale, const v
   // prompt portions: 64 rows per workgroup over key / value tiles staged in LDS (or, by a.prefill_kernel == 1,
   // 16 rows per workgroup with the key tiles shared out over four waves)
   if ((int64_t)a.T * rep <= 16 * (int64_t)a.S)
-    hipLaunchKernelGGL((window_attn_mfma_kernel<NCT, NQF, 8>), dim3(blocks, a.G), dim3(512), 0, st, a, qp, sl, vp, num_pages, op);
+    hipLaunchKernelGGL((window_attn_mfma_kernel<NCT, NQF, 8, BIAS>), dim3(blocks, a.G), dim3(512), dyn, st, a, qp, sl, vp, num_pages, op);
   else if (a.prefill_kernel == 1 || NCT > 8)
-    hipLaunchKernelGGL((window_attn_mfma_kernel<NCT, NQF, 4>), dim3(blocks, a.G), dim3(256), 0, st, a, qp, sl, vp, num_pages, op);
+    hipLaunchKernelGGL((window_attn_mfma_kernel<NCT, NQF, 4, BIAS>), dim3(blocks, a.G), dim3(256), dyn, st, a, qp, sl, vp, num_pages, op);
   else
-    hipLaunchKernelGGL((window_attn_tiled_kernel<NCT, NQF>), dim3((a.T * rep + 63) / 64 + a.S, a.G), dim3(256), 0, st, a, qp, sl,
+    hipLaunchKernelGGL((window_attn_tiled_kernel<NCT, NQF, BIAS>), dim3((a.T * rep + 63) / 64 + a.S, a.G), dim3(256), dyn, st, a, qp, sl,
                        vp, num_pages, op);
+}
+
+template <int BIAS>
+void launch_window_mfma_sized(const WindowArgs& a, const void* q, float scale, const void* vt, int num_pages, void* out,
+                              hipStream_t st) {
+  if (a.D <= 64 && a.V <= 64) launch_window_mfma<4, 2, BIAS>(a, q, scale, vt, num_pages, out, st);
+  else if (a.D <= 128 && a.V <= 128) launch_window_mfma<8, 4, BIAS>(a, q, scale, vt, num_pages, out, st);
+  else launch_window_mfma<16, 8, BIAS>(a, q, scale, vt, num_pages, out, st);
 }
 
 int heads_per_block(const WindowArgs& a) {
@@ -857,11 +929,11 @@ bool window_attn_fits(const WindowArgs& a) {
 
 void launch_window_write(const WindowArgs& a, const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v,
                          int64_t ldv, const float* qw, const float* kw, float eps, int norm_all, void* q_out, void* vt,
-                         hipStream_t st) {
+                         const float* q_head_scale, float q_temp_coef, int q_temp_every, hipStream_t st) {
   if (a.T <= 0) return;
   const size_t lds = (size_t)((a.H + a.G) * a.D + a.H + a.G) * sizeof(float);
   hipLaunchKernelGGL(window_write_kernel, dim3(a.T), dim3(256), lds, st, a, q, ldq, k, ldk, v, ldv, qw, kw, eps, norm_all,
-                     q_out, reinterpret_cast<bf16_t*>(vt));
+                     q_out, reinterpret_cast<bf16_t*>(vt), q_head_scale, q_temp_coef, q_temp_every);
 }
 
 void launch_window_pool(const WindowArgs& a, hipStream_t st) {
@@ -875,9 +947,8 @@ void launch_window_attn(const WindowArgs& a, const void* q, float scale, void* o
                         hipStream_t st) {
   if (a.T <= 0 || a.S <= 0) return;
   if (!a.f32 && vt != nullptr && a.page == 16 && a.D % 8 == 0 && a.D >= 8 && a.D <= 256 && a.V <= 256) {
-    if (a.D <= 64 && a.V <= 64) launch_window_mfma<4, 2>(a, q, scale, vt, num_pages, out, st);
-    else if (a.D <= 128 && a.V <= 128) launch_window_mfma<8, 4>(a, q, scale, vt, num_pages, out, st);
-    else launch_window_mfma<16, 8>(a, q, scale, vt, num_pages, out, st);
+    if (a.bias_kind != 0) launch_window_mfma_sized<1>(a, q, scale, vt, num_pages, out, st);
+    else launch_window_mfma_sized<0>(a, q, scale, vt, num_pages, out, st);
     return;
   }
   const int HC = heads_per_block(a);

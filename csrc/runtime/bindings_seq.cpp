@@ -351,8 +351,10 @@ void* window_vt(const OptT& vt, const Tensor& vc) {
 
 void window_write(const Tensor& q, const Tensor& k, const Tensor& v, const OptT& qw, const OptT& kw, double eps,
                   bool norm_all, const Tensor& positions, const Tensor& slots, const Tensor& inv_freq, int64_t rot_dims,
-                  const OptT& v_freq, Tensor& kc, Tensor& vc, Tensor& q_out, int64_t H, int64_t G, const OptT& vt) {
+                  const OptT& v_freq, Tensor& kc, Tensor& vc, Tensor& q_out, int64_t H, int64_t G, const OptT& vt,
+                  const OptT& q_head_scale, double q_temp_coef, int64_t q_temp_every) {
   auto a = window_common(kc, vc, c10::nullopt, c10::nullopt, H, 0);
+  TORCH_CHECK(q_temp_every >= 1, "window_write: q_temp_every >= 1");
   TORCH_CHECK(G == a.G, "window_write: kv heads");
   const int64_t T = q.size(0);
   TORCH_CHECK(act_f32(q, "q") == a.f32 && act_f32(k, "k") == a.f32 && act_f32(v, "v") == a.f32 && q.dim() == 2 &&
@@ -374,7 +376,8 @@ void window_write(const Tensor& q, const Tensor& k, const Tensor& v, const OptT&
   void* vtp = window_vt(vt, vc);
   c10::DeviceGuard guard(q.device());
   vgate::launch_window_write(a, q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), qwp, kwp,
-                             (float)eps, norm_all ? 1 : 0, q_out.data_ptr(), vtp, cur_stream());
+                             (float)eps, norm_all ? 1 : 0, q_out.data_ptr(), vtp, f32p(q_head_scale, "q_head_scale", H),
+                             (float)q_temp_coef, (int)q_temp_every, cur_stream());
 }
 
 void window_seq_meta(vgate::WindowArgs& a, const Tensor& block_tables, const Tensor& query_start) {
@@ -398,7 +401,7 @@ void window_pool(const Tensor& kc, const Tensor& vc, const OptT& kp, const OptT&
 void window_attn(const Tensor& q, const Tensor& kc, const Tensor& vc, const OptT& kp, const OptT& vp,
                  const Tensor& block_tables, const Tensor& context_lens, const Tensor& query_start, Tensor& out,
                  double scale, int64_t H, int64_t window, int64_t pool, const OptT& sink, const OptT& v_freq, const OptT& vt,
-                 int64_t prefill_kernel) {
+                 int64_t prefill_kernel, int64_t bias_kind, const OptT& bias_a, const OptT& bias_b, const OptT& gate) {
   auto a = window_common(kc, vc, kp, vp, H, pool);
   window_seq_meta(a, block_tables, query_start);
   a.context_lens = i32p(context_lens, "context_lens", a.S);
@@ -406,8 +409,30 @@ void window_attn(const Tensor& q, const Tensor& kc, const Tensor& vc, const OptT
   TORCH_CHECK(act_f32(q, "q") == a.f32 && q.dim() == 2 && q.is_contiguous() && q.size(1) == H * a.D, "window_attn: q [T, H D]");
   TORCH_CHECK(act_f32(out, "out") == a.f32 && out.dim() == 2 && out.is_contiguous() && out.size(0) == T &&
               out.size(1) == H * a.V, "window_attn: out [T, H V]");
-  TORCH_CHECK(window >= 1, "window_attn: window >= 1");
+  TORCH_CHECK(window >= 1 && window <= (1 << 30), "window_attn: window 1 .. 2^30");
   a.T = (int)T; a.window = (int)window;
+  TORCH_CHECK(bias_kind >= 0 && bias_kind <= 2, "window_attn: bias_kind 0 (none), 1 (log) or 2 (table)");
+  a.bias_kind = (int)bias_kind;
+  if (bias_kind != 0) {
+    TORCH_CHECK(pool == 0, "window_attn: a distance term and pooled blocks do not combine");
+    TORCH_CHECK(has(bias_a), "window_attn: bias_a missing");
+    if (bias_kind == 1) {
+      a.bias_a = f32p(bias_a, "bias_a", H);
+      TORCH_CHECK(has(bias_b), "window_attn: bias_b missing");
+      a.bias_b = f32p(bias_b, "bias_b", H);
+    } else {
+      TORCH_CHECK(bias_a->dim() == 2 && bias_a->size(0) == H && bias_a->size(1) >= 1 && bias_a->size(1) < (1 << 24),
+                  "window_attn: distance table [H, distances]");
+      a.bias_a = f32p(bias_a, "bias_a", -1);
+      a.bias_n = (int)bias_a->size(1);
+      a.bias_lds = (int64_t)(H / a.G) * a.bias_n * 4 <= 16 * 1024;   // beside the kernels' own tiles
+    }
+  }
+  if (has(gate)) {
+    TORCH_CHECK(act_f32(*gate, "gate") == a.f32 && gate->dim() == 2 && gate->size(0) >= T && gate->size(1) == H * a.V,
+                "window_attn: gate [T, H V] of q's dtype");
+    a.gate = gate->data_ptr(); a.ldg = gate->stride(0);
+  }
   a.sink = f32p(sink, "sink", H);
   a.v_freq = f32p(v_freq, "v_freq", a.V / 2);
   const void* vtp = window_vt(vt, vc);
@@ -418,9 +443,10 @@ void window_attn(const Tensor& q, const Tensor& kc, const Tensor& vc, const OptT
 }
 
 void linear_attn(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& g, const OptT& z, const OptT& head_decay,
-                 double tau, double q_scale, bool in_silu, const Tensor& nw, bool norm_all, bool gate_silu, Tensor& state,
+                 double tau, double q_scale, bool in_silu, const OptT& nw, bool norm_all, bool gate_silu, Tensor& state,
                  const Tensor& state_slots, const Tensor& context_lens, const Tensor& query_start, Tensor& out, double eps,
-                 Tensor& scratch, int64_t cols_per_lane) {
+                 Tensor& scratch, int64_t cols_per_lane, double k_scale, const OptT& positions, const OptT& inv_freq,
+                 int64_t rot_dims, bool rot_half) {
   vgate::LinearAttnArgs p;
   TORCH_CHECK(cols_per_lane >= 0 && cols_per_lane <= 4, "linear_attn: cols_per_lane 0 (auto), 1 or 4");
   p.cols_per_lane = (int)cols_per_lane;
@@ -445,9 +471,15 @@ void linear_attn(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor
     TORCH_CHECK(tau > 0, "linear_attn: tau > 0");
   }
   p.head_decay = f32p(head_decay, "head_decay", p.H);
-  OptT nwo(nw);
-  p.nw = f32p(nwo, "nw", norm_all ? HV : p.V);
-  p.tau = (float)tau; p.q_scale = (float)q_scale; p.eps = (float)eps;
+  p.nw = f32p(nw, "nw", norm_all ? HV : p.V);
+  p.tau = (float)tau; p.q_scale = (float)q_scale; p.k_scale = (float)k_scale; p.eps = (float)eps;
+  TORCH_CHECK(rot_dims >= 0 && rot_dims <= p.D && rot_dims % 2 == 0, "linear_attn: rot_dims even, <= key size");
+  p.rot_dims = (int)rot_dims; p.rot_half = rot_half ? 1 : 0;
+  if (rot_dims > 0) {
+    TORCH_CHECK(has(positions) && has(inv_freq) && inv_freq->numel() >= rot_dims / 2, "linear_attn: positions / inv_freq");
+    p.positions = i32p(*positions, "positions", T);
+    p.inv_freq = f32p(inv_freq, "inv_freq", -1);
+  }
   p.in_silu = in_silu; p.norm_all = norm_all; p.gate_silu = gate_silu;
   p.state = state.data_ptr<float>();
   p.S = (int)state_slots.numel();
@@ -462,7 +494,8 @@ void linear_attn(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor
   vgate::launch_linear_attn(p, (int)T, scratch.data_ptr<float>(), cur_stream());
 }
 
-void moe_route(const Tensor& z, const OptT& corr, int64_t top, double norm_eps, Tensor& idx, Tensor& wts) {
+void moe_route(const Tensor& z, const OptT& corr, int64_t top, double norm_eps, Tensor& idx, Tensor& wts, bool softmax,
+               double scale) {
   TORCH_CHECK(z.is_cuda() && z.scalar_type() == torch::kFloat32 && z.is_contiguous() && z.dim() == 2, "moe_route: z fp32 [T, E]");
   const int64_t T = z.size(0), E = z.size(1);
   TORCH_CHECK(top >= 1 && top <= E, "moe_route: top");
@@ -470,7 +503,7 @@ void moe_route(const Tensor& z, const OptT& corr, int64_t top, double norm_eps, 
   TORCH_CHECK(wts.is_cuda() && wts.scalar_type() == torch::kFloat32 && wts.is_contiguous() && wts.numel() == T * top, "moe_route: wts");
   c10::DeviceGuard guard(z.device());
   vgate::launch_moe_route(z.data_ptr<float>(), f32p(corr, "corr", E), (int)T, (int)E, (int)top, (float)norm_eps,
-                          idx.data_ptr<int32_t>(), wts.data_ptr<float>(), cur_stream());
+                          softmax ? 1 : 0, (float)scale, idx.data_ptr<int32_t>(), wts.data_ptr<float>(), cur_stream());
 }
 
 void moe_sort(const Tensor& idx, int64_t E, Tensor& rows, Tensor& pos, Tensor& off) {
@@ -485,18 +518,74 @@ void moe_sort(const Tensor& idx, int64_t E, Tensor& rows, Tensor& pos, Tensor& o
                          off.data_ptr<int32_t>(), cur_stream());
 }
 
-void moe_combine(const Tensor& y, const Tensor& pos, const Tensor& wts, Tensor& out) {
-  const int f = act_f32(y, "y");
-  TORCH_CHECK(out.dim() == 2 && out.is_contiguous() && act_f32(out, "out") == f && y.is_contiguous() && y.dim() == 2 &&
+void moe_combine(const Tensor& y, const Tensor& pos, const Tensor& wts, Tensor& out, const OptT& add) {
+  const int f = act_f32(y, "y"), of = act_f32(out, "out");
+  TORCH_CHECK(out.dim() == 2 && out.is_contiguous() && y.is_contiguous() && y.dim() == 2 &&
               y.size(1) == out.size(1), "moe_combine: y [T * top, W], out [T, W]");
+  const void* addp = nullptr;
+  if (has(add)) {
+    TORCH_CHECK(act_f32(*add, "add") == of && add->dim() == 2 && add->is_contiguous() && add->size(0) >= out.size(0) &&
+                add->size(1) == out.size(1), "moe_combine: add [T, W] of out's dtype");
+    addp = add->data_ptr();
+  }
   const int64_t T = out.size(0), W = out.size(1);
   TORCH_CHECK(T > 0 && y.size(0) % T == 0, "moe_combine: rows of y");
   const int64_t top = y.size(0) / T;
   const int32_t* pp = i32p(pos, "pos", T * top);
   OptT wo(wts);
   c10::DeviceGuard guard(y.device());
-  vgate::launch_moe_combine(y.data_ptr(), pp, f32p(wo, "wts", T * top), (int)T, (int)W, (int)top, f, out.data_ptr(),
-                            cur_stream());
+  vgate::launch_moe_combine(y.data_ptr(), pp, f32p(wo, "wts", T * top), (int)T, (int)W, (int)top, f, addp, out.data_ptr(),
+                            of, cur_stream());
+}
+
+void tanh_norm_rows(const Tensor& x, const Tensor& alpha, const Tensor& w, const Tensor& b, Tensor& y, const OptT& rows) {
+  TORCH_CHECK(x.is_cuda() && x.scalar_type() == torch::kFloat32 && x.dim() == 2 && x.stride(1) == 1, "tanh_norm_rows: x fp32 [M, n]");
+  const int yf = act_f32(y, "y");
+  TORCH_CHECK(y.dim() == 2 && y.size(1) == x.size(1), "tanh_norm_rows: y [M, n]");
+  const int64_t n = x.size(1), M = y.size(0);
+  OptT ao(alpha), wo(w), bo(b);
+  const int32_t* rp = nullptr;
+  if (has(rows)) rp = i32p(*rows, "rows", M);   // values < rows of x: row numbers of the step's batch
+  else TORCH_CHECK(x.size(0) >= M, "tanh_norm_rows: x rows");
+  c10::DeviceGuard guard(x.device());
+  vgate::launch_tanh_norm_rows(x.data_ptr<float>(), x.stride(0), rp, f32p(ao, "alpha", 1), f32p(wo, "w", n), f32p(bo, "b", n),
+                               y.data_ptr(), y.stride(0), yf, (int)M, (int)n, cur_stream());
+}
+
+void hyper_mix(Tensor& xs, const OptT& y, const OptT& mix, const OptT& out_w, const OptT& read_w, const OptT& alpha,
+               const OptT& w, const OptT& b, const OptT& h_out, const OptT& sum_out) {
+  vgate::HyperArgs a;
+  TORCH_CHECK(xs.is_cuda() && xs.scalar_type() == torch::kFloat32 && xs.dim() == 3 && xs.is_contiguous(), "hyper_mix: xs fp32 [S, T, W]");
+  a.S = (int)xs.size(0); a.T = (int)xs.size(1); a.W = (int)xs.size(2);
+  TORCH_CHECK(a.S >= 1 && a.S <= vgate::kMaxStreams, "hyper_mix: 1 .. ", vgate::kMaxStreams, " copies");
+  a.xs = xs.data_ptr<float>(); a.plane = xs.stride(0);
+  auto rows = [&](const Tensor& t, const char* name) {
+    TORCH_CHECK(t.dim() == 2 && t.is_contiguous() && t.size(0) == a.T && t.size(1) == a.W, "hyper_mix: ", name, " [T, W]");
+  };
+  if (has(y)) {
+    a.y_f32 = act_f32(*y, "y");
+    rows(*y, "y");
+    a.y = y->data_ptr();
+    TORCH_CHECK(has(mix) && has(out_w), "hyper_mix: mix / out_w come with y");
+    a.mix = f32p(mix, "mix", (int64_t)a.S * a.S);
+    a.out_w = f32p(out_w, "out_w", a.S);
+  }
+  if (has(read_w)) {
+    TORCH_CHECK(has(alpha) && has(w) && has(b) && has(h_out), "hyper_mix: alpha / w / b / h_out come with read_w");
+    a.read_w = f32p(read_w, "read_w", a.S);
+    a.alpha = f32p(alpha, "alpha", 1); a.w = f32p(w, "w", a.W); a.b = f32p(b, "b", a.W);
+    Tensor h = *h_out;
+    a.h_f32 = act_f32(h, "h_out");
+    rows(h, "h_out");
+    a.h_out = h.data_ptr();
+  }
+  if (has(sum_out)) {
+    TORCH_CHECK(sum_out->is_cuda() && sum_out->scalar_type() == torch::kFloat32, "hyper_mix: sum_out fp32");
+    rows(*sum_out, "sum_out");
+    a.sum_out = sum_out->data_ptr<float>();
+  }
+  c10::DeviceGuard guard(xs.device());
+  vgate::launch_hyper_mix(a, cur_stream());
 }
 
 }  // namespace
@@ -531,12 +620,14 @@ void bind_seq(pybind11::module& m) {
   m.def("window_write", &window_write, "q / k norm + rotation + paged key / value stores of window attention", py::arg("q"),
         py::arg("k"), py::arg("v"), py::arg("qw"), py::arg("kw"), py::arg("eps"), py::arg("norm_all"), py::arg("positions"),
         py::arg("slots"), py::arg("inv_freq"), py::arg("rot_dims"), py::arg("v_freq"), py::arg("kc"), py::arg("vc"),
-        py::arg("q_out"), py::arg("H"), py::arg("G"), py::arg("vt") = py::none());
+        py::arg("q_out"), py::arg("H"), py::arg("G"), py::arg("vt") = py::none(), py::arg("q_head_scale") = py::none(),
+        py::arg("q_temp_coef") = 0.0, py::arg("q_temp_every") = 1);
   m.def("window_pool", &window_pool, "mean key / value rows of the blocks a step completes");
   m.def("window_attn", &window_attn, "sliding-window attention with pooled blocks and an optional sink", py::arg("q"),
         py::arg("kc"), py::arg("vc"), py::arg("kp"), py::arg("vp"), py::arg("block_tables"), py::arg("context_lens"),
         py::arg("query_start"), py::arg("out"), py::arg("scale"), py::arg("H"), py::arg("window"), py::arg("pool"),
-        py::arg("sink"), py::arg("v_freq"), py::arg("vt") = py::none(), py::arg("prefill_kernel") = 0);
+        py::arg("sink"), py::arg("v_freq"), py::arg("vt") = py::none(), py::arg("prefill_kernel") = 0,
+        py::arg("bias_kind") = 0, py::arg("bias_a") = py::none(), py::arg("bias_b") = py::none(), py::arg("gate") = py::none());
   m.def("linear_attn_scratch", [](int64_t T, int64_t S, int64_t H, int64_t D, int64_t V) {
     return (int64_t)vgate::linear_attn_scratch_floats((int)T, (int)S, (int)H, (int)D, (int)V);
   }, "fp32 elements of scratch a linear_attn call over T rows and S sequences needs");
@@ -544,8 +635,14 @@ void bind_seq(pybind11::module& m) {
         py::arg("k"), py::arg("v"), py::arg("g"), py::arg("z"), py::arg("head_decay"), py::arg("tau"), py::arg("q_scale"),
         py::arg("in_silu"), py::arg("nw"), py::arg("norm_all"), py::arg("gate_silu"), py::arg("state"), py::arg("state_slots"),
         py::arg("context_lens"), py::arg("query_start"), py::arg("out"), py::arg("eps"), py::arg("scratch"),
-        py::arg("cols_per_lane") = 0);
-  m.def("moe_route", &moe_route, "sigmoid router: corrected top-k choice, normalised uncorrected weights");
+        py::arg("cols_per_lane") = 0, py::arg("k_scale") = 1.0, py::arg("positions") = py::none(),
+        py::arg("inv_freq") = py::none(), py::arg("rot_dims") = 0, py::arg("rot_half") = true);
+  m.def("moe_route", &moe_route, "sigmoid or softmax router: corrected top-k choice, normalised uncorrected weights, scaled",
+        py::arg("z"), py::arg("corr"), py::arg("top"), py::arg("norm_eps"), py::arg("idx"), py::arg("wts"),
+        py::arg("softmax") = false, py::arg("scale") = 1.0);
+  m.def("tanh_norm_rows", &tanh_norm_rows, "tanh(alpha x) * w + b over (gathered) rows");
+  m.def("hyper_mix", &hyper_mix, "write of a sublayer to the stream's copies + the next sublayer's normed read + their sum");
   m.def("moe_sort", &moe_sort, "counting sort of (token, choice) pairs by expert");
-  m.def("moe_combine", &moe_combine, "weighted sum of a token's expert rows");
+  m.def("moe_combine", &moe_combine, "weighted sum of a token's expert rows (+ a shared row)", py::arg("y"), py::arg("pos"),
+        py::arg("wts"), py::arg("out"), py::arg("add") = py::none());
 }
