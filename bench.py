@@ -358,7 +358,9 @@ def main():
     ap.add_argument("--design-compare", action="store_true",
                     help="instead of the serving benchmark: prefill / decode tokens/s of a layered hybrid design beside a "
                          "transformer of equal layer sizes (benchmarks/design_compare.py)")
-    ap.add_argument("--design", default="zadirax", choices=["zadirax", "pozalorn"], help="the design --design-compare measures")
+    ap.add_argument("--design", default="zadirax", choices=["zadirax", "pozalorn", "livitar"], help="the design --design-compare measures")
+    ap.add_argument("--design-beside", default="transformer",
+                    help="what --design-compare runs beside the design: transformer (Qwen2 layers of equal sizes) or another design")
     ap.add_argument("--design-only", action="store_true", help="--design-compare without the transformer runs")
     ap.add_argument("--design-sizes", default="1024,1536", help="widths to compare (1024, 1536)")
     ap.add_argument("--design-prefill", type=int, default=2048)
@@ -369,7 +371,7 @@ def main():
         sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "benchmarks"))
         import design_compare
         design_compare.main([int(x) for x in args.design_sizes.split(",")], args.design_prefill, args.design_batch,
-                            args.design_context, design=args.design, only_design=args.design_only)
+                            args.design_context, design=args.design, only_design=args.design_only, beside=args.design_beside)
         return
     if args.switch_interval_us > 0:
         sys.setswitchinterval(args.switch_interval_us * 1e-6)

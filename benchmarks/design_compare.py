@@ -1,9 +1,9 @@
-"""Prefill and decode throughput of a layered hybrid design (Zadirax, Pozalorn) beside the closest
-transformer family at equal layer sizes (random weights, the same number of layers), through the
-engine's own step path.
+"""Prefill and decode throughput of a layered hybrid design (Zadirax, Pozalorn, Livitar) beside the closest
+transformer family, or beside another of the designs, at equal layer sizes (random weights, the same number
+of layers), through the engine's own step path.
 
-    python bench.py --design-compare [--design zadirax|pozalorn] [--design-sizes 1024,1536]
-                    [--design-prefill 2048] [--design-batch 32] [--design-context 512]
+    python bench.py --design-compare [--design zadirax|pozalorn|livitar] [--design-beside transformer|<design>]
+                    [--design-sizes 1024,1536] [--design-prefill 2048] [--design-batch 32] [--design-context 512]
 
 Both models run teacher-forced steps (``LLMEngine.replay_step``: cache manager, step metadata, model
 forward and kernels; eager launches, nothing sampled):
@@ -78,12 +78,14 @@ def measure(model: str, overrides: dict | None, prefill: int, batch: int, contex
 _QWEN = {1024: dict(hidden_size=1024, num_heads=8, num_kv_heads=2, intermediate_size=4096, vocab_size=32000, tie_embeddings=False),
          1536: dict(hidden_size=1536, num_heads=12, num_kv_heads=2, intermediate_size=8960, vocab_size=32000, tie_embeddings=False)}
 # design -> (layers of its bench presets, "<design>-bench-<width>")
-DESIGNS = {"zadirax": 4, "pozalorn": 3}
+DESIGNS = {"zadirax": 4, "pozalorn": 3, "livitar": 3}
 
 
 def main(sizes: list[int], prefill: int = 2048, batch: int = 32, context: int = 512, design: str = "zadirax",
-         only_design: bool = False) -> dict:
+         only_design: bool = False, beside: str = "transformer") -> dict:
     layers = DESIGNS[design]
+    if beside != "transformer" and DESIGNS.get(beside) != layers:
+        raise ValueError(f"--design-beside {beside}: a design whose bench presets have {layers} layers, or transformer")
     summary = {}
     for w in sizes:
         preset = f"{design}-bench-{w}"
@@ -91,11 +93,15 @@ def main(sizes: list[int], prefill: int = 2048, batch: int = 32, context: int = 
         print(json.dumps({"width": w, "model": preset, **a}), flush=True)
         if only_design:
             continue
-        b = measure("qwen2.5-1.5b", dict(_QWEN[w], num_layers=layers), prefill, batch, context, 32000)
-        print(json.dumps({"width": w, "model": f"qwen2 ({layers} layers, equal width)", **b}), flush=True)
+        if beside == "transformer":
+            b = measure("qwen2.5-1.5b", dict(_QWEN[w], num_layers=layers), prefill, batch, context, 32000)
+            print(json.dumps({"width": w, "model": f"qwen2 ({layers} layers, equal width)", **b}), flush=True)
+        else:
+            b = measure(f"{beside}-bench-{w}", None, prefill, batch, context, 32000)
+            print(json.dumps({"width": w, "model": f"{beside}-bench-{w}", **b}), flush=True)
         summary[str(w)] = {"prefill_ratio": round(a["prefill_tok_s"] / b["prefill_tok_s"], 3),
                            "decode_ratio": round(a["decode_tok_s"] / b["decode_tok_s"], 3)}
-    line = {"metric": f"{design} vs transformer at equal layer sizes, tokens/s ratio ({layers} layers, eager steps)",
+    line = {"metric": f"{design} vs {beside} at equal layer sizes, tokens/s ratio ({layers} layers, eager steps)",
             "prefill_tokens": prefill, "decode_batch": batch, "decode_context": context, "ratios": summary}
     print(json.dumps(line), flush=True)
     return line

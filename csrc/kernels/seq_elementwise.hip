@@ -183,6 +183,60 @@ __global__ __launch_bounds__(256) void hyper_mix_kernel(HyperArgs a) {
   }
 }
 
+// one wave per token, lane l holding the scores of experts l, l + 64, .. (E <= 64 RPL): `top` (<= 64) rounds of
+// a wave-wide arg-max over the corrected scores (lowest index wins a tie)
+constexpr int RPL = 8;
+__global__ __launch_bounds__(256) void moe_route_wave_kernel(const float* __restrict__ z, const float* __restrict__ corr,
+                                                             int T, int E, int top, float norm_eps, int softmax, float scale,
+                                                             int32_t* __restrict__ idx, float* __restrict__ wts) {
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (t >= T) return;  // (wave-uniform)
+  const float* zr = z + (int64_t)t * E;
+  float s[RPL], v[RPL];
+  float zmax = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < RPL; ++j) {
+    const int e = lane + 64 * j;
+    s[j] = e < E ? zr[e] : -INFINITY;
+    zmax = fmaxf(zmax, s[j]);
+  }
+  float den = 1.f;
+  if (softmax) {  // scores over all experts: exp(z - max) / sum
+    zmax = wave_reduce_max(zmax);
+    float part = 0.f;
+#pragma unroll
+    for (int j = 0; j < RPL; ++j) part += lane + 64 * j < E ? expf(s[j] - zmax) : 0.f;
+    den = wave_reduce_sum(part);
+  }
+#pragma unroll
+  for (int j = 0; j < RPL; ++j) {
+    const int e = lane + 64 * j;
+    s[j] = softmax ? expf(s[j] - zmax) / den : sigm(s[j]);
+    v[j] = e < E ? s[j] + (corr ? corr[e] : 0.f) : -INFINITY;
+  }
+  float sum = 0.f, mine = 0.f;
+  for (int c = 0; c < top; ++c) {
+    float bv = -INFINITY, bs = 0.f;
+    int bi = 0x7fffffff;
+#pragma unroll
+    for (int j = 0; j < RPL; ++j)   // (ascending index inside a lane: strict > keeps the lowest)
+      if (lane + 64 * j < E && (bi == 0x7fffffff || v[j] > bv)) { bv = v[j]; bi = lane + 64 * j; bs = s[j]; }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, 64), os = __shfl_xor(bs, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi))) { bv = ov; bi = oi; bs = os; }
+    }
+#pragma unroll
+    for (int j = 0; j < RPL; ++j)
+      if (lane + 64 * j == bi) v[j] = -INFINITY, s[j] = 0.f;   // taken (only its owner's copy matters)
+    if (lane == 0) idx[(int64_t)t * top + c] = bi;
+    if (lane == c) mine = bs;
+    sum += bs;
+  }
+  if (lane < top) wts[(int64_t)t * top + lane] = mine * (1.f / (sum + norm_eps)) * scale;
+}
+
 // one thread per token: `top` rounds of arg-max over the corrected scores (lowest index wins a tie)
 __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ z, const float* __restrict__ corr,
                                                         int T, int E, int top, float norm_eps, int softmax, float scale,
@@ -300,6 +354,11 @@ void launch_gated_residual(float* x, const void* y1, const void* g1, int64_t ldg
 void launch_moe_route(const float* z, const float* corr, int T, int E, int top, float norm_eps, int softmax, float scale,
                       int32_t* idx, float* wts, hipStream_t st) {
   if (T <= 0) return;
+  if (E <= 64 * RPL && top <= 64) {
+    hipLaunchKernelGGL(moe_route_wave_kernel, dim3((T + 3) / 4), dim3(256), 0, st, z, corr, T, E, top, norm_eps, softmax,
+                       scale, idx, wts);
+    return;
+  }
   hipLaunchKernelGGL(moe_route_kernel, dim3((T + 63) / 64), dim3(64), 0, st, z, corr, T, E, top, norm_eps, softmax, scale,
                      idx, wts);
 }

@@ -181,7 +181,7 @@ void launch_tanh_norm_rows(const float* x, int64_t ldx, const int32_t* rows, con
 //   y given:      xs[t] <- sum_s mix[s][t] xs[s] + out_w[t] * y      (all copies at once from the old ones)
 //   read_w given: h_out = tanh(alpha[0] * sum_s read_w[s] xs[s]) * w + b   (from the new copies)
 //   sum_out given: the sum of the new copies
-constexpr int kMaxStreams = 8;
+constexpr int kMaxStreams = 16;
 struct HyperArgs {
   float* xs = nullptr; int64_t plane = 0;
   const void* y = nullptr; int y_f32 = 0;

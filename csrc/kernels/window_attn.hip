@@ -394,6 +394,23 @@ __device__ __forceinline__ float bias_of(const WindowArgs& a, const float* btab,
   const int idx = bo + min(n, a.bias_n - 1);
   return a.bias_lds ? btab[idx] : a.bias_a[(int64_t)g * rep * a.bias_n + idx] * LOG2E;
 }
+// the terms of a lane's 4 x 2 scores of one tile (keys c0 and c0 + 16), asked for together, before the softmax's
+// arithmetic, and whether the key is visible or not (a negative distance reads entry 0). all_far (wave-uniform):
+// every key of the tile is at least the table's last distance away from every row of the wave.
+__device__ __forceinline__ void bias_tile(const WindowArgs& a, const float* btab, int g, int rep, const float* bw,
+                                          const float* bx, const int* bo, const float* bfar, const int* hi, int c0,
+                                          bool all_far, float* bt0, float* bt1) {
+  if (a.bias_kind == 2 && all_far) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) bt0[i] = bt1[i] = bfar[i];
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    bt0[i] = bias_of(a, btab, g, rep, bw[i], bx[i], bo[i], hi[i] - c0);
+    bt1[i] = bias_of(a, btab, g, rep, bw[i], bx[i], bo[i], hi[i] - c0 - 16);
+  }
+}
 __device__ __forceinline__ float gate_of(const bf16_t* grow, int col) { return 1.f / (1.f + __expf(-bf2f(grow[col]))); }
 
 // NCT: 16-column tiles of the value (V <= 16 NCT); NQF: 32-wide fragments of a query row (D <= 32 NQF).
@@ -445,7 +462,7 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
   // C-layout rows of this lane: row0 + 4 lg + i; what each sees: tokens [lo, hi], pooled blocks [0, nbv)
   int hi[4], lo[4], nbv[4];
   float m[4], lsum[4];
-  float bw[BIAS ? 4 : 1], bx[BIAS ? 4 : 1];
+  float bw[BIAS ? 4 : 1], bx[BIAS ? 4 : 1], bfar[BIAS ? 4 : 1];
   int bo[BIAS ? 4 : 1];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -455,7 +472,10 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
     hi[i] = ok ? p : -1;
     lo[i] = p - a.window + 1;
     nbv[i] = (ok && P > 0) ? max(0, lo[i]) / P : 0;
-    if (BIAS) bias_row(a, g, rep, r, ok, bw[i], bx[i], bo[i]);
+    if (BIAS) {
+      bias_row(a, g, rep, r, ok, bw[i], bx[i], bo[i]);
+      bfar[i] = a.bias_kind == 2 ? bias_of(a, btab, g, rep, 0.f, 0.f, bo[i], a.bias_n - 1) : 0.f;
+    }
     const bool sk = ok && a.sink != nullptr && wv == 0;  // the sink counts once
     m[i] = sk ? a.sink[g * rep + r % rep] * 1.4426950408889634f : -INFINITY;
     lsum[i] = (sk && lr == 0) ? 1.f : 0.f;
@@ -511,16 +531,14 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
     }
     float al[4];
     const int c0 = kbase + lr, c1 = kbase + 16 + lr;
+    float bt0[BIAS ? 4 : 1], bt1[BIAS ? 4 : 1];
+    if (BIAS) bias_tile(a, btab, g, rep, bw, bx, bo, bfar, hi, c0, kbase + 31 <= pmin - (a.bias_n - 1), bt0, bt1);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const bool vis0 = pooled ? c0 < nbv[i] : (c0 >= lo[i] && c0 <= hi[i]);
       const bool vis1 = pooled ? c1 < nbv[i] : (c1 >= lo[i] && c1 <= hi[i]);
-      float v0 = vis0 ? s0[i] * scale_log2e : -INFINITY;
-      float v1 = vis1 ? s1[i] * scale_log2e : -INFINITY;
-      if (BIAS) {  // (never with pooled tiles)
-        if (vis0) v0 += bias_of(a, btab, g, rep, bw[i], bx[i], bo[i], hi[i] - c0);
-        if (vis1) v1 += bias_of(a, btab, g, rep, bw[i], bx[i], bo[i], hi[i] - c1);
-      }
+      const float v0 = vis0 ? fmaf(s0[i], scale_log2e, BIAS ? bt0[i] : 0.f) : -INFINITY;
+      const float v1 = vis1 ? fmaf(s1[i], scale_log2e, BIAS ? bt1[i] : 0.f) : -INFINITY;
       const float mnew = fmaxf(m[i], group16_max(fmaxf(v0, v1)));
       const float ms = (mnew == -INFINITY) ? 0.f : mnew;  // a row that has seen no key yet
       al[i] = exp2f(m[i] - ms);
@@ -678,7 +696,10 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(WindowArgs a, co
   const int nqf = (D + 31) >> 5, nct = (V + 15) >> 4, d8 = D >> 3;
   for (int e = tid; e < 2 * 32 * DP / 8; e += 256) reinterpret_cast<uint4*>(&kl[0][0][0])[e] = make_uint4(0, 0, 0, 0);
   for (int e = tid; e < 2 * 16 * NCT * VP / 8; e += 256) reinterpret_cast<uint4*>(&vl[0][0][0])[e] = make_uint4(0, 0, 0, 0);
-  if (BIAS) bias_stage(a, btab, g, rep, tid, 256);  // (the barrier before the first tile covers it)
+  if (BIAS) {
+    bias_stage(a, btab, g, rep, tid, 256);
+    __syncthreads();  // the rows' set-up below reads the staged table
+  }
   bf16x8 qf[NQF];
   {
     const int r = row0 + lr;
@@ -689,7 +710,7 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(WindowArgs a, co
   }
   int hi[4], lo[4], nbv[4];
   float m[4], lsum[4];
-  float bw[BIAS ? 4 : 1], bx[BIAS ? 4 : 1];
+  float bw[BIAS ? 4 : 1], bx[BIAS ? 4 : 1], bfar[BIAS ? 4 : 1];
   int bo[BIAS ? 4 : 1];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -699,7 +720,10 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(WindowArgs a, co
     hi[i] = ok ? p : -1;
     lo[i] = p - a.window + 1;
     nbv[i] = (ok && P > 0) ? max(0, lo[i]) / P : 0;
-    if (BIAS) bias_row(a, g, rep, r, ok, bw[i], bx[i], bo[i]);
+    if (BIAS) {
+      bias_row(a, g, rep, r, ok, bw[i], bx[i], bo[i]);
+      bfar[i] = a.bias_kind == 2 ? bias_of(a, btab, g, rep, 0.f, 0.f, bo[i], a.bias_n - 1) : 0.f;
+    }
     const bool sk = ok && a.sink != nullptr;
     m[i] = sk ? a.sink[g * rep + r % rep] * 1.4426950408889634f : -INFINITY;
     lsum[i] = (sk && lr == 0) ? 1.f : 0.f;
@@ -722,16 +746,14 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(WindowArgs a, co
   auto softmax_tile = [&](const f32x4& s0, const f32x4& s1, int kbase, bool pooled) {
     float al[4];
     const int c0 = kbase + lr, c1 = kbase + 16 + lr;
+    float bt0[BIAS ? 4 : 1], bt1[BIAS ? 4 : 1];
+    if (BIAS) bias_tile(a, btab, g, rep, bw, bx, bo, bfar, hi, c0, kbase + 31 <= pminw - (a.bias_n - 1), bt0, bt1);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const bool vis0 = pooled ? c0 < nbv[i] : (c0 >= lo[i] && c0 <= hi[i]);
       const bool vis1 = pooled ? c1 < nbv[i] : (c1 >= lo[i] && c1 <= hi[i]);
-      float v0 = vis0 ? s0[i] * scale_log2e : -INFINITY;
-      float v1 = vis1 ? s1[i] * scale_log2e : -INFINITY;
-      if (BIAS) {  // (never with pooled tiles)
-        if (vis0) v0 += bias_of(a, btab, g, rep, bw[i], bx[i], bo[i], hi[i] - c0);
-        if (vis1) v1 += bias_of(a, btab, g, rep, bw[i], bx[i], bo[i], hi[i] - c1);
-      }
+      const float v0 = vis0 ? fmaf(s0[i], scale_log2e, BIAS ? bt0[i] : 0.f) : -INFINITY;
+      const float v1 = vis1 ? fmaf(s1[i], scale_log2e, BIAS ? bt1[i] : 0.f) : -INFINITY;
       const float mnew = fmaxf(m[i], group16_max(fmaxf(v0, v1)));
       const float ms = (mnew == -INFINITY) ? 0.f : mnew;
       al[i] = exp2f(m[i] - ms);

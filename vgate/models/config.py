@@ -372,8 +372,9 @@ HYBRID_PRESETS = {
     # tests / CPU smoke: odd sizes on purpose
     "livitar-tiny": lambda: _livitar_preset("livitar-tiny", 88, 300, 1, 4, 2, 24, 5, 2, 40, 56, streams=3, ret_heads=3, buckets_far=50),
     # slices at the layer sizes of real models beside a transformer of equal width (benchmarks/design_compare.py)
-    "livitar-bench-1024": lambda: _livitar_preset("livitar-bench-1024", 1024, 32000, 1, 8, 2, 128, 8, 2, 2048, 2048),
-    "livitar-bench-1536": lambda: _livitar_preset("livitar-bench-1536", 1536, 32000, 1, 12, 2, 128, 16, 4, 2240, 2240),
+    # (the chosen experts and the shared one together are as wide as the dense feed-forward of the other bench presets)
+    "livitar-bench-1024": lambda: _livitar_preset("livitar-bench-1024", 1024, 32000, 1, 8, 2, 128, 8, 2, 1024, 2048),
+    "livitar-bench-1536": lambda: _livitar_preset("livitar-bench-1536", 1536, 32000, 1, 12, 2, 128, 16, 4, 1792, 1792),
     # layer sizes of a ~1.5B model (the width, head size, feed-forward and vocabulary of qwen2.5-1.5b)
     "zadirax-1.5b": lambda: _zadirax_preset("zadirax-1.5b", 1536, 151936, 14, 12, 128, 8960, 32, 4, 2240, 512, 768, 64),
 }

@@ -44,7 +44,7 @@ def _C():
 
 ACT_NONE, ACT_SILU_MUL, ACT_CLAMPED_GLU, ACT_TANH, ACT_GELU_TANH_MUL = 0, 1, 2, 3, 4
 BIAS_NONE, BIAS_LOG, BIAS_TABLE = 0, 1, 2   # distance term of an attention score (see window_attn)
-MAX_STREAMS = 8             # copies of the residual stream hyper_mix takes
+MAX_STREAMS = 16            # copies of the residual stream hyper_mix takes
 LINEAR_ATTN_MAX_DIM = 256   # key channels per head the recurrence kernel keeps in registers (csrc/kernels/linear_attn.hip)
 
 
