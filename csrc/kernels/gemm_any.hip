@@ -8,6 +8,9 @@
 // activation in the epilogue).
 //   bf16: 64 x 64 block tile, 4 waves of 2 x 2 v_mfma_f32_16x16x32_bf16 tiles, operands read as 16-B
 //         fragments straight from global memory (both operands are k-contiguous rows), fp32 accumulate.
+//         Large aligned products (hundreds of rows, wide outputs: the expert GEMMs of a prompt portion):
+//         128 x 128 block tile (a weight pair: 128 x 64 of each matrix), 4 waves of 4 x 4 MFMA tiles, k-steps of
+//         32 staged through two LDS buffers, the next step's loads in flight during the current step's MFMAs.
 //   fp32: 64 x 64 x 16 LDS-tiled FMA kernel, 4 x 4 outputs per thread, k ascending.
 #include <cstdlib>
 
@@ -19,17 +22,17 @@ namespace {
 
 constexpr int BM = 64, BN = 64;
 
-__device__ __forceinline__ bool locate_tile(const AnyGemmArgs& p, int by, int& grp, int& r0, int& rend) {
+__device__ __forceinline__ bool locate_tile(const AnyGemmArgs& p, int by, int& grp, int& r0, int& rend, int bm = BM) {
   if (p.group_off == nullptr) {
-    grp = 0; r0 = by * BM; rend = p.M;
+    grp = 0; r0 = by * bm; rend = p.M;
     return r0 < p.M;
   }
   int base = 0;
   for (int g = 0; g < p.groups; ++g) {
     const int a = p.group_off[g], b = p.group_off[g + 1];
-    const int nt = (b - a + BM - 1) / BM;
+    const int nt = (b - a + bm - 1) / bm;
     if (by < base + nt) {
-      grp = g; r0 = a + (by - base) * BM; rend = b;
+      grp = g; r0 = a + (by - base) * bm; rend = b;
       return true;
     }
     base += nt;
@@ -197,6 +200,103 @@ __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(AnyGemmArgs p) {
     }
 }
 
+// LDS-tiled form. Host-checked: K, the row strides and the batch strides are multiples of 8 elements, the bases
+// 16-B aligned, K >= 8. Block tile 128 rows x 128 weight rows (DUAL: rows 0..63 of the tile are W's, 64..127 the
+// same columns of W2, so a lane holds gate and up of one output); wave (wm, wn) owns rows 64 wm .. and 4 x 4 MFMA
+// tiles. A k-step's 128 x 32 A and weight tiles are two 16-B pieces per thread each; rows past the group's end
+// read the tile's first row and columns past N the last one (both dropped at the store), k past K reads a
+// clamped address and zeroes the A piece.
+constexpr int LM = 128, LKS = 32, LPAD = LKS + 8;
+template <int DUAL>
+__global__ __launch_bounds__(256) void gemm_any_lds_kernel(AnyGemmArgs p) {
+  constexpr int WN = DUAL ? 64 : 128;  // columns of each weight matrix per block
+  __shared__ __attribute__((aligned(16))) bf16_t As[2][LM][LPAD];
+  __shared__ __attribute__((aligned(16))) bf16_t Ws[2][128][LPAD];
+  int grp, r0, rend;
+  if (!locate_tile(p, blockIdx.y, grp, r0, rend, LM)) return;
+  const int64_t b = blockIdx.z;
+  const int64_t wsel = (p.group_off != nullptr) ? grp : b;
+  const int n0 = blockIdx.x * WN;
+  const int tid = threadIdx.x, l = tid & 63, wv = tid >> 6;
+  const int wm = wv & 1, wn = wv >> 1, lr = l & 15, lg = l >> 4;
+  const bf16_t* A = reinterpret_cast<const bf16_t*>(p.a) + b * p.a_bs;
+  const bf16_t* W = reinterpret_cast<const bf16_t*>(p.w) + wsel * p.w_bs;
+  const bf16_t* W2 = DUAL ? reinterpret_cast<const bf16_t*>(p.w2) + wsel * p.w_bs : nullptr;
+  const int K = p.K;
+  const int kq = (tid & 3) * 8;  // this thread's quarter of a k-step
+  const bf16_t* asrc[2];
+  const bf16_t* wsrc[2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int row = (tid >> 2) + 64 * u;
+    const int m = r0 + row < rend ? r0 + row : r0;
+    asrc[u] = A + (int64_t)(p.a_rows ? p.a_rows[m] : m) * p.lda;
+    const int n = min(n0 + (DUAL ? (row & 63) : row), p.N - 1);
+    wsrc[u] = ((DUAL && row >= 64) ? W2 : W) + (int64_t)n * p.ldw;
+  }
+  f32x4 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  uint4 ar[2], wr[2];
+  auto fetch = [&](int k0) {
+    const int k = k0 + kq, kk = min(k, K - 8);
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      ar[u] = ld16(asrc[u] + kk);
+      wr[u] = ld16(wsrc[u] + kk);
+      if (k >= K) ar[u] = make_uint4(0, 0, 0, 0);  // a zero A piece zeroes the product
+    }
+  };
+  auto stage = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int row = (tid >> 2) + 64 * u;
+      *reinterpret_cast<uint4*>(&As[buf][row][kq]) = ar[u];
+      *reinterpret_cast<uint4*>(&Ws[buf][row][kq]) = wr[u];
+    }
+  };
+  fetch(0);
+  stage(0);
+  __syncthreads();
+  int buf = 0;
+  // a buffer is rewritten one step later, after the barrier that every wave reaches only when it has read it
+  for (int k0 = 0; k0 < K; k0 += LKS) {
+    const bool more = k0 + LKS < K;
+    if (more) fetch(k0 + LKS);
+    bf16x8 af[4], wf[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) af[i] = as_bf16x8(*reinterpret_cast<const uint4*>(&As[buf][wm * 64 + i * 16 + lr][8 * lg]));
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int wrow = DUAL ? (j >> 1) * 64 + wn * 32 + (j & 1) * 16 + lr : wn * 64 + j * 16 + lr;
+      wf[j] = as_bf16x8(*reinterpret_cast<const uint4*>(&Ws[buf][wrow][8 * lg]));
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = mfma16(af[i], wf[j], acc[i][j]);
+    if (more) stage(buf ^ 1);
+    __syncthreads();
+    buf ^= 1;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < (DUAL ? 2 : 4); ++j) {
+      const int n = n0 + (DUAL ? wn * 32 : wn * 64) + j * 16 + lr;
+      if (n >= p.N) continue;
+      const float bias = p.bias ? p.bias[n] : 0.f;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int m = r0 + wm * 64 + i * 16 + 4 * lg + e;
+        if (m >= rend) continue;
+        store_out(p, b, m, n, epi_val(p, acc[i][j][e] + bias, DUAL ? acc[i][j + 2][e] : 0.f));
+      }
+    }
+}
+
 template <typename T>
 __device__ __forceinline__ float ldf(const T* q);
 template <>
@@ -279,6 +379,15 @@ __global__ __launch_bounds__(256) void gemm_any_fma_kernel(AnyGemmArgs p) {
   }
 }
 
+// "1": large products through the LDS-tiled kernel (default); "0": the direct-fragment kernels only
+bool lds_tiles() {
+  static const bool v = [] {
+    const char* e = getenv("VGATE_GEMM_ANY_LDS");
+    return e == nullptr || e[0] != '0';
+  }();
+  return v;
+}
+
 bool simple_only() {
   static const bool v = [] {
     const char* e = getenv("VGATE_GEMM_ANY_FMA");
@@ -306,7 +415,11 @@ void launch_gemm_any(const AnyGemmArgs& g, hipStream_t st) {
                     g.w_bs % 8 == 0 && a16(g.a) && a16(g.w) && (!dual || a16(g.w2));
     const bool wide = al && g.N >= 512 && g.M >= 256;  // enough 64 x 128 tiles to fill the chip
     const dim3 gridw((g.N + 127) / 128, mt, g.batch);
-    if (dual && wide) hipLaunchKernelGGL((gemm_any_mfma_kernel<1, true, 4>), gridw, block, 0, st, g);
+    if (wide && g.M >= 1024 && lds_tiles()) {  // enough 128-row tiles
+      const int mt128 = (g.M + LM - 1) / LM + (g.group_off ? g.groups : 0);
+      if (dual) hipLaunchKernelGGL((gemm_any_lds_kernel<1>), dim3((g.N + 63) / 64, mt128, g.batch), block, 0, st, g);
+      else hipLaunchKernelGGL((gemm_any_lds_kernel<0>), dim3((g.N + 127) / 128, mt128, g.batch), block, 0, st, g);
+    } else if (dual && wide) hipLaunchKernelGGL((gemm_any_mfma_kernel<1, true, 4>), gridw, block, 0, st, g);
     else if (wide) hipLaunchKernelGGL((gemm_any_mfma_kernel<0, true, 4>), gridw, block, 0, st, g);
     else if (dual && al) hipLaunchKernelGGL((gemm_any_mfma_kernel<1, true, 2>), grid, block, 0, st, g);
     else if (dual) hipLaunchKernelGGL((gemm_any_mfma_kernel<1, false, 2>), grid, block, 0, st, g);

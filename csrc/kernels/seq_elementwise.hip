@@ -140,24 +140,25 @@ __global__ __launch_bounds__(256) void tanh_norm_rows_kernel(const float* __rest
     stx(y, (int64_t)m * ldy + c, y_f32, fmaf(tanhf(al * x[src * ldx_ + c]), w[c], b[c]));
 }
 
-// one thread per (token, column): the S copies of the element are read, mixed and written by the same thread
+// one thread per (token, column): the S <= MS copies of the element are read, mixed and written by the same thread
+template <int MS>
 __global__ __launch_bounds__(256) void hyper_mix_kernel(HyperArgs a) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= (int64_t)a.T * a.W) return;
   const int c = (int)(i % a.W);
   const int S = a.S;
-  float x[kMaxStreams];
+  float x[MS];
 #pragma unroll
-  for (int s = 0; s < kMaxStreams; ++s) x[s] = s < S ? a.xs[s * a.plane + i] : 0.f;
+  for (int s = 0; s < MS; ++s) x[s] = s < S ? a.xs[s * a.plane + i] : 0.f;
   if (a.y != nullptr) {
     const float yv = ldx(a.y, i, a.y_f32);
-    float nx[kMaxStreams];
+    float nx[MS];
 #pragma unroll
-    for (int t = 0; t < kMaxStreams; ++t) {
+    for (int t = 0; t < MS; ++t) {
       float v = 0.f;
       if (t < S) {
 #pragma unroll
-        for (int s = 0; s < kMaxStreams; ++s)
+        for (int s = 0; s < MS; ++s)
           if (s < S) v = fmaf(a.mix[s * S + t], x[s], v);
         v = fmaf(a.out_w[t], yv, v);
         a.xs[t * a.plane + i] = v;
@@ -165,19 +166,19 @@ __global__ __launch_bounds__(256) void hyper_mix_kernel(HyperArgs a) {
       nx[t] = v;
     }
 #pragma unroll
-    for (int s = 0; s < kMaxStreams; ++s) x[s] = nx[s];
+    for (int s = 0; s < MS; ++s) x[s] = nx[s];
   }
   if (a.read_w != nullptr) {
     float u = 0.f;
 #pragma unroll
-    for (int s = 0; s < kMaxStreams; ++s)
+    for (int s = 0; s < MS; ++s)
       if (s < S) u = fmaf(a.read_w[s], x[s], u);
     stx(a.h_out, i, a.h_f32, fmaf(tanhf(a.alpha[0] * u), a.w[c], a.b[c]));
   }
   if (a.sum_out != nullptr) {
     float u = 0.f;
 #pragma unroll
-    for (int s = 0; s < kMaxStreams; ++s)
+    for (int s = 0; s < MS; ++s)
       if (s < S) u += x[s];
     a.sum_out[i] = u;
   }
@@ -372,7 +373,10 @@ void launch_tanh_norm_rows(const float* x, int64_t ldx_, const int32_t* rows, co
 void launch_hyper_mix(const HyperArgs& a, hipStream_t st) {
   const int64_t tot = (int64_t)a.T * a.W;
   if (tot <= 0 || a.S <= 0) return;
-  hipLaunchKernelGGL(hyper_mix_kernel, dim3((unsigned)((tot + 255) / 256)), dim3(256), 0, st, a);
+  const dim3 grid((unsigned)((tot + 255) / 256));
+  if (a.S <= 2) hipLaunchKernelGGL(hyper_mix_kernel<2>, grid, dim3(256), 0, st, a);
+  else if (a.S <= 4) hipLaunchKernelGGL(hyper_mix_kernel<4>, grid, dim3(256), 0, st, a);
+  else hipLaunchKernelGGL(hyper_mix_kernel<kMaxStreams>, grid, dim3(256), 0, st, a);
 }
 
 void launch_moe_sort(const int32_t* idx, int T, int E, int top, int32_t* rows, int32_t* pos, int32_t* off,
