@@ -92,16 +92,23 @@ __device__ __forceinline__ bf16x8 load_frag(const bf16_t* rowp, int k, int K, bo
 // their MFMAs, so the loads of a wave overlap.
 // NJ: 16-column tiles per wave (2: 64-column block tile; 4: 128-column block tile for wide outputs, which
 // loads 1.5x fewer fragment bytes per MFMA)
+// A tile with at most 32 rows (an expert's few rows of a decode step) on the aligned 64-column form: the two
+// waves that would split the rows split the k range instead (k-steps of 64 in turn, so each weight fragment is
+// loaded by one wave only and a wave's dependent chain of loads is half as long) and add up through LDS.
 template <int DUAL, bool AL, int NJ>
 __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(AnyGemmArgs p) {
+  constexpr bool KS = AL && NJ == 2;
+  __shared__ f32x4 red[KS ? 2 : 1][KS ? (DUAL ? 8 : 4) : 1][KS ? 64 : 1];
   int grp, r0, rend;
   if (!locate_tile(p, blockIdx.y, grp, r0, rend)) return;
+  const bool ks = KS && rend - r0 <= 32;  // (workgroup-uniform)
   const int64_t b = blockIdx.z;
   const int64_t wsel = (p.group_off != nullptr) ? grp : b;
   const int n0 = blockIdx.x * (32 * NJ);
   const int l = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int wm = wv & 1, wn = wv >> 1;
   const int lr = l & 15, lk = 8 * (l >> 4);
+  const int mrow = ks ? 0 : wm * 32;  // first row of this wave
   const bf16_t* A = reinterpret_cast<const bf16_t*>(p.a) + b * p.a_bs;
   const bf16_t* W = reinterpret_cast<const bf16_t*>(p.w) + wsel * p.w_bs;
   const bf16_t* W2 = DUAL ? reinterpret_cast<const bf16_t*>(p.w2) + wsel * p.w_bs : nullptr;
@@ -109,7 +116,7 @@ __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(AnyGemmArgs p) {
   bool aval[2];
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
-    const int m = r0 + wm * 32 + i * 16 + lr;
+    const int m = r0 + mrow + i * 16 + lr;
     aval[i] = m < rend;
     const int src = aval[i] ? (p.a_rows ? p.a_rows[m] : m) : 0;
     arow[i] = A + (int64_t)src * p.lda;
@@ -135,7 +142,7 @@ __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(AnyGemmArgs p) {
   if (AL) {
     const uint4 zero = make_uint4(0, 0, 0, 0);
     const int K = p.K;
-    for (int k0 = 0; k0 < K; k0 += 64) {
+    for (int k0 = ks ? 64 * wm : 0; k0 < K; k0 += ks ? 128 : 64) {
       uint4 av[2][2], wv_[2][NJ], uv[2][NJ];
 #pragma unroll
       for (int st = 0; st < 2; ++st) {
@@ -184,6 +191,26 @@ __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(AnyGemmArgs p) {
         if (DUAL) acc2[i][j] = mfma16(af[i], b2[j], acc2[i][j]);
       }
   }
+  if (KS && ks) {  // the k halves of a wave pair: wm 1 hands its sums to wm 0
+    if (wm == 1) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+          red[KS ? wn : 0][KS ? 2 * i + j : 0][KS ? l : 0] = acc[i][j];
+          if (DUAL) red[KS ? wn : 0][KS ? 4 + 2 * i + j : 0][KS ? l : 0] = acc2[i][j];
+        }
+    }
+    __syncthreads();
+    if (wm == 1) return;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        acc[i][j] += red[KS ? wn : 0][KS ? 2 * i + j : 0][KS ? l : 0];
+        if (DUAL) acc2[i][j] += red[KS ? wn : 0][KS ? 4 + 2 * i + j : 0][KS ? l : 0];
+      }
+  }
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -193,7 +220,7 @@ __global__ __launch_bounds__(256) void gemm_any_mfma_kernel(AnyGemmArgs p) {
       const float bias = p.bias ? p.bias[n] : 0.f;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const int m = r0 + wm * 32 + i * 16 + 4 * (l >> 4) + e;
+        const int m = r0 + mrow + i * 16 + 4 * (l >> 4) + e;
         if (m >= rend) continue;
         store_out(p, b, m, n, epi_val(p, acc[i][j][e] + bias, DUAL ? acc2[i][j][e] : 0.f));
       }

@@ -298,10 +298,10 @@ class WindowAttention:
         if self.qk_norm != "none":
             if m.get("qk_norm_weight", True):
                 self.qw, self.kw = _f32(tensors["q.norm"], dev), _f32(tensors["k.norm"], dev)
-            else:
-                n = self.D if self.qk_norm == "head" else None
-                self.qw = torch.ones(n or self.H * self.D, dtype=torch.float32, device=dev)
-                self.kw = torch.ones(n or self.G * self.D, dtype=torch.float32, device=dev)
+            else:   # a norm without a weight: ones
+                per_head = self.qk_norm == "head"
+                self.qw = torch.ones(self.D if per_head else self.H * self.D, dtype=torch.float32, device=dev)
+                self.kw = torch.ones(self.D if per_head else self.G * self.D, dtype=torch.float32, device=dev)
         self.sink = _f32(tensors["sink"], dev) if m.get("sink") else None
         self.head_temp = _f32(tensors["temp"], dev) if m.get("head_temp") else None
         qt = m.get("q_temp") or {}
@@ -331,11 +331,10 @@ class WindowAttention:
         out = {"q": (H * D, width), "k": (G * D, width), "v": (G * V, width), "o": (width, H * V)}
         if spec.get("bias"):
             out.update({"q.b": (H * D,), "k.b": (G * D,), "v.b": (G * V,)})
-        if not spec.get("qk_norm_weight", True):
-            pass
-        elif spec.get("qk_norm", "none") == "head":
+        weighted = spec.get("qk_norm_weight", True)
+        if weighted and spec.get("qk_norm", "none") == "head":
             out.update({"q.norm": (D,), "k.norm": (D,)})
-        elif spec.get("qk_norm") == "all":
+        elif weighted and spec.get("qk_norm") == "all":
             out.update({"q.norm": (H * D,), "k.norm": (G * D,)})
         if spec.get("gate"):
             out["g"] = (H * V, width)
