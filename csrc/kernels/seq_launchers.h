@@ -110,6 +110,9 @@ struct WindowArgs {
   int bias_kind = 0, bias_n = 0, bias_lds = 0;   // bias_lds: the MFMA kernels stage a workgroup's heads' table in LDS
   const float* bias_a = nullptr; const float* bias_b = nullptr;
   const void* gate = nullptr; int64_t ldg = 0;   // [T][H * V] rows (activation dtype): out *= sigmoid(gate); null: none
+  // decoded tokens, MFMA kernel: parts > 1 workgroups share a 16-row tile's keys and leave partial results in
+  // part_o [parts][G][tiles][16][16 NCT] / part_ml [parts][G][tiles][16][2] for a merge launch
+  int parts = 1; float* part_o = nullptr; float* part_ml = nullptr;
   const int32_t* positions = nullptr;   // [T]
   const int32_t* slots = nullptr;       // [T] page * tokens-per-page + offset of each token (-1: padding)
   const int32_t* block_tables = nullptr; const int32_t* context_lens = nullptr; const int32_t* query_start = nullptr;
@@ -117,6 +120,11 @@ struct WindowArgs {
   void* kp = nullptr; void* vp = nullptr;  // [pages][G][npool][D | V]
 };
 size_t window_attn_lds_bytes(const WindowArgs& a, int heads_per_block);
+// how many workgroups share a decoded token's key tiles (1: no split; only the bf16 MFMA kernel splits), and the
+// fp32 scratch elements window_attn then needs
+int window_attn_parts(int T, int S, int H, int G, int D, int V, int f32, int page);
+int window_attn_nct(int D, int V);   // 16-column value tiles of the MFMA kernel instantiation for these head sizes
+size_t window_attn_part_floats(int T, int S, int H, int G, int D, int V, int parts);
 bool window_attn_fits(const WindowArgs& a);   // sizes the kernels' LDS and register budgets take
 // q / k norm (qw, kw null: none; norm_all: one norm over the whole projection) + rotation + paged stores; q_out [T][H * D];
 // the query of head h at position p is multiplied by q_head_scale[h] (null: 1) * (1 + q_temp_coef ln(floor((p + 1) / q_temp_every) + 1));

@@ -476,7 +476,7 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
       bias_row(a, g, rep, r, ok, bw[i], bx[i], bo[i]);
       bfar[i] = a.bias_kind == 2 ? bias_of(a, btab, g, rep, 0.f, 0.f, bo[i], a.bias_n - 1) : 0.f;
     }
-    const bool sk = ok && a.sink != nullptr && wv == 0;  // the sink counts once
+    const bool sk = ok && a.sink != nullptr && wv == 0 && blockIdx.z == 0;  // the sink counts once
     m[i] = sk ? a.sink[g * rep + r % rep] * 1.4426950408889634f : -INFINITY;
     lsum[i] = (sk && lr == 0) ? 1.f : 0.f;
   }
@@ -490,7 +490,10 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
 #pragma unroll
   for (int ct = 0; ct < NCT; ++ct) O[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int32_t* bt = a.block_tables + (int64_t)s * a.max_blocks;
-  for (int ti = wv; ti < ntiles; ti += NW) {
+  // a.parts > 1 (decoded tokens of long contexts): blockIdx.z is one of several workgroups that share the key tiles
+  // of these 16 rows; each leaves its merged (max, sum, weighted values) in scratch for window_attn_merge_kernel
+  const int nparts = a.parts > 1 ? a.parts : 1;
+  for (int ti = blockIdx.z * NW + wv; ti < ntiles; ti += NW * nparts) {
     const bool pooled = ti < ntp;  // wave-uniform
     int kbase, pg0 = 0, pg1 = 0;
     const bf16_t* k0p;
@@ -629,6 +632,19 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
   // eight waves (decoded tokens) share the epilogue out: wave w finishes the column tiles ct = w, w + NW, ..;
   // with four (prompt portions) wave 0 finishes all of them: the shared form costs four registers there, which
   // is the step from four waves per SIMD to three (measured 167 us against 109 us)
+  if (a.parts > 1) {  // (workgroup-uniform) hand the partial result on: the merge kernel finishes the rows
+    const int64_t slot = ((int64_t)blockIdx.z * G + g) * gridDim.x + blockIdx.x;
+    float* po = a.part_o + slot * (16 * 16 * NCT);
+    for (int e = threadIdx.x; e < 16 * 16 * NCT; e += 64 * NW) po[e] = (&mrg_o[0][0])[e];
+    if (wv == 0 && lr == 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        a.part_ml[(slot * 16 + 4 * lg + i) * 2] = m[i];
+        a.part_ml[(slot * 16 + 4 * lg + i) * 2 + 1] = lsum[i];
+      }
+    }
+    return;
+  }
   constexpr bool SHARE = NW > 4;
   if (!SHARE && wv != 0) return;
   const int vrot = a.v_freq != nullptr ? 2 * (V / 2) : 0;
@@ -656,6 +672,61 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
       }
       if (ok && ct < nct && col < V) orow[col] = f2bf(grow != nullptr ? y * gate_of(grow, col) : y);
     }
+  }
+}
+
+// The rows of one 16-row tile from the partial results of a.parts workgroups: M = max of the parts' maxima (log2
+// units), sums and weighted values rescaled by 2^(M_p - M) and added in part order, then the epilogue of the kernel
+// above (normalise, turn back, gate, store). vs: the row stride of the parts' weighted values.
+__global__ __launch_bounds__(256) void window_attn_merge_kernel(WindowArgs a, int vs, bf16_t* __restrict__ out) {
+  const int V = a.V, G = a.G, H = a.H, rep = H / G, g = blockIdx.y;
+  int s = -1, tile = 0, base = 0;
+  for (int i = 0; i < a.S; ++i) {
+    const int nt = ((a.query_start[i + 1] - a.query_start[i]) * rep + 15) / 16;
+    if ((int)blockIdx.x < base + nt) { s = i; tile = blockIdx.x - base; break; }
+    base += nt;
+  }
+  if (s < 0) return;
+  const int t0 = a.query_start[s], ntok = a.query_start[s + 1] - t0;
+  const int pos0 = a.context_lens[s] - ntok, nrows = ntok * rep;
+  const int vrot = a.v_freq != nullptr ? 2 * (V / 2) : 0;
+  // blockIdx.z: which four rows of the tile
+  for (int e = threadIdx.x; e < 4 * V; e += blockDim.x) {
+    const int rr = 4 * blockIdx.z + e / V, col = e % V, r = tile * 16 + rr;
+    if (r >= nrows) continue;
+    constexpr int MAXP = 8;  // (window_attn_parts() gives at most eight)
+    float pm[MAXP], pl[MAXP], po[MAXP], M = -INFINITY;
+#pragma unroll
+    for (int p = 0; p < MAXP; ++p) {  // all parts' loads asked for together
+      const int64_t slot = ((int64_t)min(p, a.parts - 1) * G + g) * gridDim.x + blockIdx.x;
+      pm[p] = p < a.parts ? a.part_ml[(slot * 16 + rr) * 2] : -INFINITY;
+      pl[p] = a.part_ml[(slot * 16 + rr) * 2 + 1];
+      po[p] = a.part_o[slot * (16 * vs) + rr * vs + col];
+      M = fmaxf(M, pm[p]);
+    }
+    float L = 0.f, y = 0.f, yo = 0.f;  // yo: the pair's other column (turned values)
+    const int colo = col ^ 1;
+#pragma unroll
+    for (int p = 0; p < MAXP; ++p) {
+      const float f = exp2f(pm[p] - M);  // a part that saw no key (or is none): max -inf, factor 0
+      L = fmaf(pl[p], f, L);
+      y = fmaf(po[p], f, y);
+      if (col < vrot && p < a.parts) {
+        const int64_t slot = ((int64_t)p * G + g) * gridDim.x + blockIdx.x;
+        yo = fmaf(a.part_o[slot * (16 * vs) + rr * vs + colo], f, yo);
+      }
+    }
+    const float inv = 1.f / L;
+    y *= inv;
+    if (col < vrot) {
+      const float ang = -(float)(pos0 + r / rep) * a.v_freq[col >> 1];
+      const float cs = cosf(ang), sn = sinf(ang);
+      yo *= inv;
+      y = (col & 1) ? (y * cs + yo * sn) : (y * cs - yo * sn);
+    }
+    const int64_t t = t0 + r / rep, h = g * rep + r % rep;
+    if (a.gate != nullptr) y *= gate_of(reinterpret_cast<const bf16_t*>(a.gate) + t * a.ldg + h * V, col);
+    out[(t * H + h) * V + col] = f2bf(y);
   }
 }
 
@@ -912,8 +983,12 @@ void launch_window_mfma(const WindowArgs& a, const void* q, float scale, const v
   // few rows per sequence (decoded tokens): few workgroups, so eight waves each stream the keys of 16 rows;
   // prompt portions: 64 rows per workgroup over key / value tiles staged in LDS (or, by a.prefill_kernel == 1,
   // 16 rows per workgroup with the key tiles shared out over four waves)
-  if ((int64_t)a.T * rep <= 16 * (int64_t)a.S)
-    hipLaunchKernelGGL((window_attn_mfma_kernel<NCT, NQF, 8, BIAS>), dim3(blocks, a.G), dim3(512), dyn, st, a, qp, sl, vp, num_pages, op);
+  if ((int64_t)a.T * rep <= 16 * (int64_t)a.S) {
+    const int parts = a.parts > 1 ? a.parts : 1;
+    hipLaunchKernelGGL((window_attn_mfma_kernel<NCT, NQF, 8, BIAS>), dim3(blocks, a.G, parts), dim3(512), dyn, st, a, qp, sl, vp,
+                       num_pages, op);
+    if (parts > 1) hipLaunchKernelGGL(window_attn_merge_kernel, dim3(blocks, a.G, 4), dim3(256), 0, st, a, 16 * NCT, op);
+  }
   else if (a.prefill_kernel == 1 || NCT > 8)
     hipLaunchKernelGGL((window_attn_mfma_kernel<NCT, NQF, 4, BIAS>), dim3(blocks, a.G), dim3(256), dyn, st, a, qp, sl, vp, num_pages, op);
   else
@@ -921,11 +996,16 @@ void launch_window_mfma(const WindowArgs& a, const void* q, float scale, const v
                        vp, num_pages, op);
 }
 
+}  // namespace
+int window_attn_nct(int D, int V);
+namespace {
+
 template <int BIAS>
 void launch_window_mfma_sized(const WindowArgs& a, const void* q, float scale, const void* vt, int num_pages, void* out,
                               hipStream_t st) {
-  if (a.D <= 64 && a.V <= 64) launch_window_mfma<4, 2, BIAS>(a, q, scale, vt, num_pages, out, st);
-  else if (a.D <= 128 && a.V <= 128) launch_window_mfma<8, 4, BIAS>(a, q, scale, vt, num_pages, out, st);
+  const int nct = window_attn_nct(a.D, a.V);  // (the scratch of a split launch is sized by the same rule)
+  if (nct == 4) launch_window_mfma<4, 2, BIAS>(a, q, scale, vt, num_pages, out, st);
+  else if (nct == 8) launch_window_mfma<8, 4, BIAS>(a, q, scale, vt, num_pages, out, st);
   else launch_window_mfma<16, 8, BIAS>(a, q, scale, vt, num_pages, out, st);
 }
 
@@ -938,6 +1018,22 @@ int heads_per_block(const WindowArgs& a) {
 }
 
 }  // namespace
+
+// Decoded tokens on the MFMA kernel: how many workgroups share the key tiles of a 16-row tile (1: no split) so that
+// the launch has about two workgroups of eight waves per CU, and the scratch floats their partial results take.
+int window_attn_parts(int T, int S, int H, int G, int D, int V, int f32, int page) {
+  const int rep = H / G;
+  if (f32 || page != 16 || D % 8 != 0 || D < 8 || D > 256 || V > 256 || (int64_t)T * rep > 16 * (int64_t)S) return 1;
+  const int wg = ((T * rep + 15) / 16 + S) * G;
+  const int parts = 512 / (wg > 0 ? wg : 1);
+  return parts < 2 ? 1 : (parts > 8 ? 8 : parts);
+}
+int window_attn_nct(int D, int V) { return (D <= 64 && V <= 64) ? 4 : ((D <= 128 && V <= 128) ? 8 : 16); }
+size_t window_attn_part_floats(int T, int S, int H, int G, int D, int V, int parts) {
+  const int rep = H / G;
+  const size_t slots = (size_t)parts * G * ((T * rep + 15) / 16 + S);
+  return parts > 1 ? slots * 16 * (16 * window_attn_nct(D, V) + 2) : 0;
+}
 
 size_t window_attn_lds_bytes(const WindowArgs& a, int HC) {
   return ((size_t)HC * (a.D + 1) + (size_t)KT * (a.D + 1) + (size_t)KT * (a.V + 1) + HC * KT + 3 * HC + (size_t)HC * a.V) *

@@ -401,7 +401,8 @@ void window_pool(const Tensor& kc, const Tensor& vc, const OptT& kp, const OptT&
 void window_attn(const Tensor& q, const Tensor& kc, const Tensor& vc, const OptT& kp, const OptT& vp,
                  const Tensor& block_tables, const Tensor& context_lens, const Tensor& query_start, Tensor& out,
                  double scale, int64_t H, int64_t window, int64_t pool, const OptT& sink, const OptT& v_freq, const OptT& vt,
-                 int64_t prefill_kernel, int64_t bias_kind, const OptT& bias_a, const OptT& bias_b, const OptT& gate) {
+                 int64_t prefill_kernel, int64_t bias_kind, const OptT& bias_a, const OptT& bias_b, const OptT& gate,
+                 int64_t parts, const OptT& part_scratch) {
   auto a = window_common(kc, vc, kp, vp, H, pool);
   window_seq_meta(a, block_tables, query_start);
   a.context_lens = i32p(context_lens, "context_lens", a.S);
@@ -436,6 +437,19 @@ void window_attn(const Tensor& q, const Tensor& kc, const Tensor& vc, const OptT
   a.sink = f32p(sink, "sink", H);
   a.v_freq = f32p(v_freq, "v_freq", a.V / 2);
   const void* vtp = window_vt(vt, vc);
+  if (parts > 1) {  // only what window_attn_parts() allows for this launch, with its scratch
+    TORCH_CHECK(vtp != nullptr && parts == vgate::window_attn_parts((int)T, a.S, a.H, a.G, a.D, a.V, a.f32, a.page),
+                "window_attn: parts must be window_attn_split()'s for this step");
+    const size_t need = vgate::window_attn_part_floats((int)T, a.S, a.H, a.G, a.D, a.V, (int)parts);
+    TORCH_CHECK(has(part_scratch) && part_scratch->is_cuda() && part_scratch->scalar_type() == torch::kFloat32 &&
+                part_scratch->is_contiguous() && (size_t)part_scratch->numel() >= need, "window_attn: part_scratch fp32 with ",
+                need, " elements");
+    const int nct = vgate::window_attn_nct(a.D, a.V);
+    const size_t slots = need / (16 * (16 * nct + 2));
+    a.parts = (int)parts;
+    a.part_o = part_scratch->data_ptr<float>();
+    a.part_ml = a.part_o + slots * 16 * 16 * nct;
+  }
   TORCH_CHECK(prefill_kernel == 0 || prefill_kernel == 1, "window_attn: prefill_kernel 0 or 1");
   a.prefill_kernel = (int)prefill_kernel;
   c10::DeviceGuard guard(q.device());
@@ -627,7 +641,12 @@ void bind_seq(pybind11::module& m) {
         py::arg("kc"), py::arg("vc"), py::arg("kp"), py::arg("vp"), py::arg("block_tables"), py::arg("context_lens"),
         py::arg("query_start"), py::arg("out"), py::arg("scale"), py::arg("H"), py::arg("window"), py::arg("pool"),
         py::arg("sink"), py::arg("v_freq"), py::arg("vt") = py::none(), py::arg("prefill_kernel") = 0,
-        py::arg("bias_kind") = 0, py::arg("bias_a") = py::none(), py::arg("bias_b") = py::none(), py::arg("gate") = py::none());
+        py::arg("bias_kind") = 0, py::arg("bias_a") = py::none(), py::arg("bias_b") = py::none(), py::arg("gate") = py::none(),
+        py::arg("parts") = 1, py::arg("part_scratch") = py::none());
+  m.def("window_attn_split", [](int64_t T, int64_t S, int64_t H, int64_t G, int64_t D, int64_t V, bool f32, int64_t page) {
+    const int parts = vgate::window_attn_parts((int)T, (int)S, (int)H, (int)G, (int)D, (int)V, f32 ? 1 : 0, (int)page);
+    return std::make_pair((int64_t)parts, (int64_t)vgate::window_attn_part_floats((int)T, (int)S, (int)H, (int)G, (int)D, (int)V, parts));
+  }, "workgroups that share a decoded token's key tiles in window_attn, and the fp32 scratch elements they need");
   m.def("linear_attn_scratch", [](int64_t T, int64_t S, int64_t H, int64_t D, int64_t V) {
     return (int64_t)vgate::linear_attn_scratch_floats((int)T, (int)S, (int)H, (int)D, (int)V);
   }, "fp32 elements of scratch a linear_attn call over T rows and S sequences needs");

@@ -45,6 +45,7 @@ def _C():
 ACT_NONE, ACT_SILU_MUL, ACT_CLAMPED_GLU, ACT_TANH, ACT_GELU_TANH_MUL = 0, 1, 2, 3, 4
 BIAS_NONE, BIAS_LOG, BIAS_TABLE = 0, 1, 2   # distance term of an attention score (see window_attn)
 MAX_STREAMS = 16            # copies of the residual stream hyper_mix takes
+WINDOW_SPLIT = os.environ.get("VGATE_WINDOW_SPLIT", "1") == "1"   # "0": one workgroup per decoded 16-row tile
 LINEAR_ATTN_MAX_DIM = 256   # key channels per head the recurrence kernel keeps in registers (csrc/kernels/linear_attn.hip)
 
 
@@ -493,8 +494,14 @@ def window_attn(q, kc, vc, kp, vp, block_tables, context_lens, query_start, out,
     the MFMA kernels (``prefill_kernel``: which one prompt portions take, 0 = tiles staged in LDS for 64 rows,
     1 = 16 rows per workgroup with the tiles shared out over its waves)."""
     if q.is_cuda:
+        parts, scratch = 1, None
+        if vt is not None and WINDOW_SPLIT:   # decoded tokens of the MFMA kernel: several workgroups per 16-row tile
+            parts, n = _C().window_attn_split(q.shape[0], block_tables.shape[0], H, kc.shape[1], kc.shape[3], vc.shape[3],
+                                              kc.dtype == torch.float32, kc.shape[2])
+            if parts > 1:
+                scratch = torch.empty(n, dtype=torch.float32, device=q.device)
         _C().window_attn(q, kc, vc, kp, vp, block_tables, context_lens, query_start, out, scale, H, window, pool, sink, v_freq, vt,
-                         prefill_kernel, bias_kind, bias_a, bias_b, gate)
+                         prefill_kernel, bias_kind, bias_a, bias_b, gate, parts, scratch)
         return
     G, page, D, V = kc.shape[1], kc.shape[2], kc.shape[3], vc.shape[3]
     rep = H // G
