@@ -2,8 +2,10 @@
 // rotated key part (rot) shared by all heads. The per-head key and value up-projections are absorbed
 // into the query and the output (q' = W_uk^T q, out = W_uv (sum_j p_j c_j)), so prompt portions and
 // single decoded tokens run the same kernel on the cached rows alone:
-//   score(t, h, j) = scale * (q'[t][h] . c_j + rope(q_rot[t][h]) . k_rot_j),   j <= position(t)
+//   score(t, h, j) = scale * (q'[t][h] . c_j + rope(q_rot[t][h]) . k_rot_j),   0 <= position(t) - j < window
 //   ol[t][h]       = sum_j softmax_j(score) c_j
+// A sink (one logit per head) only enters the softmax denominator: the running max starts at it, the sum at 1.
+// Key tiles sit at absolute positions whatever the window's start, so a row's sums keep their order.
 // latent_write: RMS norm of the latent (fp32 statistics) + interleaved-pair rotation of the shared key
 // part + the paged store, one launch. Angles are position * inv_freq in fp32 with full-range sin / cos.
 // latent_attn, fp32 caches (and shapes the MFMA kernel does not take): one workgroup per (token, group
@@ -101,7 +103,8 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(LatentArgs a, const vo
                                                            int max_blocks, int page,
                                                            const int32_t* __restrict__ context_lens,
                                                            const int32_t* __restrict__ query_start, int S,
-                                                           void* __restrict__ ol) {
+                                                           void* __restrict__ ol, int window,
+                                                           const float* __restrict__ sink) {
   extern __shared__ float lds[];
   const int E = a.rank + a.rot, EP = E + 1;
   float* qs = lds;                  // [HC][EP]
@@ -119,6 +122,7 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(LatentArgs a, const vo
   }
   const int s = lo;
   const int nkeys = context_lens[s] - (query_start[s + 1] - t) + 1;
+  const int first = max(0, nkeys - window);  // the oldest key the token sees
   const int h0 = blockIdx.y * HC;
   const int nh = min(HC, H - h0);
   const int tid = threadIdx.x;
@@ -126,18 +130,23 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(LatentArgs a, const vo
     const int h = e / E, c = e % E;
     qs[h * EP + c] = ldx(qa, ((int64_t)t * H + h0 + h) * E + c, a.f32);
   }
-  if (tid < HC) { mrun[tid] = -INFINITY; lrun[tid] = 0.f; alpha[tid] = 1.f; }
+  if (tid < HC) {
+    const bool sk = sink != nullptr && tid < nh;
+    mrun[tid] = sk ? sink[h0 + tid] : -INFINITY;
+    lrun[tid] = sk ? 1.f : 0.f;
+    alpha[tid] = 1.f;
+  }
   float acc[MAXACC];
 #pragma unroll
   for (int i = 0; i < MAXACC; ++i) acc[i] = 0.f;
   const int32_t* bt = block_tables + (int64_t)s * max_blocks;
-  for (int j0 = 0; j0 < nkeys; j0 += KT) {
+  for (int j0 = (first / KT) * KT; j0 < nkeys; j0 += KT) {
     __syncthreads();  // previous tile fully consumed (and q / running stats written)
     for (int e = tid; e < KT * E; e += 256) {
       const int jj = e / E, c = e % E;
       const int kj = j0 + jj;
       float v = 0.f;
-      if (kj < nkeys) {
+      if (kj < nkeys && kj >= first) {
         const int64_t row = (int64_t)bt[kj / page] * page + kj % page;
         v = ldx(a.cache, row * E + c, a.f32);
       }
@@ -156,7 +165,7 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(LatentArgs a, const vo
         for (int c = c0; c < c1; ++c) d = fmaf(qp[c], kp[c], d);
       }
       d += __shfl_xor(d, 1, 64);
-      if (on && half == 0) sc[h * KT + jj] = (j0 + jj < nkeys) ? d * scale : -INFINITY;
+      if (on && half == 0) sc[h * KT + jj] = (j0 + jj < nkeys && j0 + jj >= first) ? d * scale : -INFINITY;
     }
     __syncthreads();
     if (tid < nh) {
@@ -164,13 +173,13 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(LatentArgs a, const vo
       float m1 = m0;
       for (int jj = 0; jj < KT; ++jj) m1 = fmaxf(m1, sc[tid * KT + jj]);
       const float al = expf(m0 - m1);  // m0 = -inf on the first tile: 0
-      float l = lrun[tid] * al;
+      float l = 0.f;  // the tile's own sum first: the running sum takes one rounding per tile, not per key
       for (int jj = 0; jj < KT; ++jj) {
         const float pj = expf(sc[tid * KT + jj] - m1);
         sc[tid * KT + jj] = pj;
         l += pj;
       }
-      mrun[tid] = m1; lrun[tid] = l; alpha[tid] = al;
+      mrun[tid] = m1; lrun[tid] = fmaf(lrun[tid], al, l); alpha[tid] = al;
     }
     __syncthreads();
 #pragma unroll
@@ -178,11 +187,11 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(LatentArgs a, const vo
       const int o = tid + i * 256;
       if (o < nh * a.rank) {
         const int h = o / a.rank, c = o % a.rank;
-        float v = acc[i] * alpha[h];
+        float v = 0.f;
         const float* pp = sc + h * KT;
 #pragma unroll
         for (int jj = 0; jj < KT; ++jj) v = fmaf(pp[jj], ks[jj * EP + c], v);
-        acc[i] = v;
+        acc[i] = fmaf(acc[i], alpha[h], v);
       }
     }
   }
@@ -248,7 +257,8 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentArgs a, con
                                                                 const int32_t* __restrict__ context_lens,
                                                                 const int32_t* __restrict__ query_start, int S,
                                                                 const bf16_t* __restrict__ cache_t,
-                                                                bf16_t* __restrict__ ol) {
+                                                                bf16_t* __restrict__ ol, int window,
+                                                                const float* __restrict__ sink) {
   __shared__ __attribute__((aligned(16))) bf16_t pl[4][16][40];
   __shared__ float mrg_m[4][16], mrg_l[4][16];
   __shared__ float mrg_o[16][16 * NCT];  // split mode: the merged weighted latent of the 16 rows
@@ -279,22 +289,26 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentArgs a, con
     for (int kk = 0; kk < NQF; ++kk) qf[kk] = frag16(qrow, 32 * kk + 8 * lg, E, ok && kk < nqf);
   }
   // C-layout rows of this lane: row0 + 4 lg + i; keys visible to each
-  int limit[4];
+  int limit[4], lowest[4];
+  float m[4], lsum[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r = row0 + 4 * lg + i;
-    limit[i] = r < nrows ? pos0 + r / H + 1 : 1;
+    const bool ok = r < nrows;
+    limit[i] = ok ? pos0 + r / H + 1 : 0;   // keys [lowest, limit); a row past the last sees none
+    lowest[i] = max(0, limit[i] - window);
+    const bool sk = ok && sink != nullptr && (!split || wv == 0);  // the sink counts once
+    m[i] = sk ? sink[r % H] * 1.4426950408889634f : -INFINITY;
+    lsum[i] = (sk && lr == 0) ? 1.f : 0.f;
   }
   const int last = min(row0 + 15, nrows - 1);
   const int kmax = pos0 + last / H + 1;  // wave-uniform
-  float m[4], lsum[4];
+  const int kmin = max(0, pos0 + row0 / H + 1 - window) & ~31;  // first tile any row of the wave sees
   f32x4 O[NCT];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) { m[i] = -INFINITY; lsum[i] = 0.f; }
 #pragma unroll
   for (int ct = 0; ct < NCT; ++ct) O[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int32_t* bt = block_tables + (int64_t)s * max_blocks;
-  for (int j0 = split ? 32 * wv : 0; j0 < kmax; j0 += split ? 128 : 32) {
+  for (int j0 = kmin + (split ? 32 * wv : 0); j0 < kmax; j0 += split ? 128 : 32) {
     int pg0 = bt[j0 >> 4];
     int pg1 = (j0 + 16 < kmax) ? bt[(j0 >> 4) + 1] : pg0;
     pg0 = min(max(pg0, 0), num_pages - 1);
@@ -323,8 +337,8 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentArgs a, con
     float al[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float v0 = (j0 + lr < limit[i]) ? s0[i] * scale_log2e : -INFINITY;
-      const float v1 = (j0 + 16 + lr < limit[i]) ? s1[i] * scale_log2e : -INFINITY;
+      const float v0 = (j0 + lr < limit[i] && j0 + lr >= lowest[i]) ? s0[i] * scale_log2e : -INFINITY;
+      const float v1 = (j0 + 16 + lr < limit[i] && j0 + 16 + lr >= lowest[i]) ? s1[i] * scale_log2e : -INFINITY;
       const float mnew = fmaxf(m[i], group16_max(fmaxf(v0, v1)));
       const float ms = (mnew == -INFINITY) ? 0.f : mnew;  // a row that has seen no key yet (split mode)
       al[i] = exp2f(m[i] - ms);
@@ -366,13 +380,14 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentArgs a, con
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int r = 4 * lg + i;
-      float M = mrg_m[0][r];  // wave 0 always holds key 0: finite
+      float M = mrg_m[0][r];
 #pragma unroll
       for (int w = 1; w < 4; ++w) M = fmaxf(M, mrg_m[w][r]);
+      const float Ms = (M == -INFINITY) ? 0.f : M;  // (rows past the sequence's last)
       float L = 0.f;
 #pragma unroll
-      for (int w = 0; w < 4; ++w) L += mrg_l[w][r] * exp2f(mrg_m[w][r] - M);
-      f[i] = exp2f(m[i] - M);     // a wave that saw no key: exp2(-inf) = 0
+      for (int w = 0; w < 4; ++w) L += mrg_l[w][r] * exp2f(mrg_m[w][r] - Ms);  // a wave that saw no key: l = 0, exp2(-inf) = 0
+      f[i] = exp2f(m[i] - Ms);
       lsum[i] = L;                // the merged row sum (the same in every lane of the row)
       m[i] = M;
     }
@@ -414,12 +429,12 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentArgs a, con
 template <int NCT, int NQF>
 void launch_mfma(const LatentArgs& a, const void* qa, int H, float scale, const int32_t* block_tables, int max_blocks,
                  int num_pages, const int32_t* context_lens, const int32_t* query_start, int S, const void* cache_t,
-                 void* ol, hipStream_t st) {
+                 void* ol, int window, const float* sink, hipStream_t st) {
   const int blocks = (a.T * H + 63) / 64 + S;
   hipLaunchKernelGGL((latent_attn_mfma_kernel<NCT, NQF>), dim3(blocks), dim3(256), 0, st, a,
                      reinterpret_cast<const bf16_t*>(qa), H, scale * 1.4426950408889634f, block_tables, max_blocks,
                      num_pages, context_lens, query_start, S, reinterpret_cast<const bf16_t*>(cache_t),
-                     reinterpret_cast<bf16_t*>(ol));
+                     reinterpret_cast<bf16_t*>(ol), window, sink);
 }
 
 }  // namespace
@@ -438,12 +453,12 @@ void launch_latent_qrope(const LatentArgs& a, const void* q, int H, int dim, voi
 
 void launch_latent_attn(const LatentArgs& a, const void* qa, int H, float scale, const int32_t* block_tables,
                         int max_blocks, int page, const int32_t* context_lens, const int32_t* query_start, int S,
-                        void* ol, const void* cache_t, int num_pages, hipStream_t st) {
+                        void* ol, const void* cache_t, int num_pages, int window, const float* sink, hipStream_t st) {
   if (a.T <= 0 || S <= 0) return;
   const int E = a.rank + a.rot;
   if (!a.f32 && cache_t != nullptr && page == 16 && a.rank <= 512 && E <= 640 && E % 8 == 0 && E >= 8) {
 #define VG_LAT(NCT, NQF) launch_mfma<NCT, NQF>(a, qa, H, scale, block_tables, max_blocks, num_pages, context_lens, \
-                                               query_start, S, cache_t, ol, st)
+                                               query_start, S, cache_t, ol, window, sink, st)
     if (a.rank <= 128 && E <= 192) VG_LAT(8, 6);
     else if (a.rank <= 256 && E <= 384) VG_LAT(16, 12);
     else VG_LAT(32, 20);
@@ -454,7 +469,7 @@ void launch_latent_attn(const LatentArgs& a, const void* qa, int H, float scale,
   while (HC > 1 && (HC * a.rank > 256 * MAXACC || (size_t)(HC + KT) * (E + 1) * 4 > 56 * 1024)) --HC;
   const size_t lds = ((size_t)(HC + KT) * (E + 1) + HC * KT + 3 * HC) * sizeof(float);
   hipLaunchKernelGGL(latent_attn_kernel, dim3(a.T, (H + HC - 1) / HC), dim3(256), lds, st, a, qa, H, HC, scale,
-                     block_tables, max_blocks, page, context_lens, query_start, S, ol);
+                     block_tables, max_blocks, page, context_lens, query_start, S, ol, window, sink);
 }
 
 }  // namespace vgate

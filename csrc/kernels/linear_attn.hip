@@ -5,7 +5,12 @@
 // silu on q, k and v, optionally rotary positions on the leading rot_dims entries of every q / k head
 // (entry i paired with i + rot_dims / 2, or 2i with 2i + 1; angle = position * inv_freq in fp32) and a key
 // scale after them, then an RMS norm of o (per head, or over the concatenated heads; with or without a
-// weight) and an output gate silu(g) or sigmoid(g). Key and value sizes may differ. Three launches:
+// weight) and an output gate silu(g) or sigmoid(g). Key and value sizes may differ.
+// Variants: the decay exp(-exp(z_t)); with a bonus u [H][D] the state is read BEFORE its update and the current
+// token's own outer product enters the output through u,
+//   o_t = (S_(t-1) + diag(u) k_t v_t^T)^T (q_scale q_t),   then   S_t = diag(a_t) S_(t-1) + k_t v_t^T
+// (PRE instantiations of the scan: the prepared vector's fourth entry is u k); a per-head norm whose weight has one
+// entry per output channel. Three launches:
 //   prep   (token, head) parallel: the fp32 per-channel triples {a, k_scale k, q_scale q} and the values.
 //   scan   the recurrence. Column v of S depends on no other column, so a head's value columns are split
 //          into slices of 8 NC and every (sequence, head, slice) is one wave: lane = (key group of eight,
@@ -61,8 +66,12 @@ __global__ __launch_bounds__(256) void linear_prep_kernel(LinearAttnArgs p, floa
       q = first ? q * cs - qo * sn : q * cs + qo * sn;
       k = first ? k * cs - ko * sn : k * cs + ko * sn;
     }
-    const float a = p.z != nullptr ? expf(log_sigmoid(p.z[(int64_t)t * p.ldz + e]) * inv_tau) : p.head_decay[e / p.D];
-    vec[(int64_t)t * HD + e] = make_float4(a, k * p.k_scale, q * p.q_scale, 0.f);
+    float a;
+    if (p.z == nullptr) a = p.head_decay[e / p.D];
+    else if (p.decay_exp) a = expf(-expf(p.z[(int64_t)t * p.ldz + e]));
+    else a = expf(log_sigmoid(p.z[(int64_t)t * p.ldz + e]) * inv_tau);
+    k *= p.k_scale;
+    vec[(int64_t)t * HD + e] = make_float4(a, k, q * p.q_scale, p.bonus != nullptr ? p.bonus[e] * k : 0.f);
   }
   for (int e = threadIdx.x; e < HV; e += blockDim.x) {
     const float v = ldx(p.v, (int64_t)t * p.ldv + e, p.f32);
@@ -90,7 +99,7 @@ __device__ __forceinline__ bool locate_chunk(const LinearAttnArgs& p, int CH, in
   return false;
 }
 
-template <int DQ, int TC, int NC, int MODE>
+template <int DQ, int TC, int NC, int MODE, bool PRE>
 __global__ __launch_bounds__(64) void linear_scan_kernel(LinearAttnArgs p, const float4* __restrict__ vec,
                                                           const float* __restrict__ vals, float* __restrict__ oraw,
                                                           int CH, float* __restrict__ cstate, float* __restrict__ cdecay) {
@@ -180,11 +189,12 @@ __global__ __launch_bounds__(64) void linear_scan_kernel(LinearAttnArgs p, const
       for (int n = 0; n < NC; ++n) { vv[n] = lvv[buf][i][cl + 8 * n]; o[n] = 0.f; }
 #pragma unroll
       for (int j = 0; j < DQ; ++j) {
-        const float4 x = tv[j];  // {a, k, q}: one LDS read serves the lane's NC columns
+        const float4 x = tv[j];  // {a, k, q, u k}: one LDS read serves the lane's NC columns
 #pragma unroll
         for (int n = 0; n < NC; ++n) {
+          if (PRE && MODE != SCAN_LOCAL) o[n] = fmaf(x.z, fmaf(x.w, vv[n], S[j][n]), o[n]);  // the state before its update
           S[j][n] = fmaf(x.y, vv[n], x.x * S[j][n]);
-          if (MODE != SCAN_LOCAL) o[n] = fmaf(x.z, S[j][n], o[n]);
+          if (!PRE && MODE != SCAN_LOCAL) o[n] = fmaf(x.z, S[j][n], o[n]);
         }
         if (MODE == SCAN_LOCAL) A[j] *= x.x;
       }
@@ -279,26 +289,34 @@ __global__ __launch_bounds__(256) void linear_finish_kernel(LinearAttnArgs p, co
     for (int c = lane; c < V; c += 64) ss = fmaf(o[h * V + c], o[h * V + c], ss);
     ss = wave_reduce_sum(ss);
     const float inv = 1.f / sqrtf(ss / (float)V + p.eps);
-    for (int c = lane; c < V; c += 64) emit(h * V + c, o[h * V + c] * inv * (p.nw != nullptr ? p.nw[c] : 1.f));
+    for (int c = lane; c < V; c += 64)
+      emit(h * V + c, o[h * V + c] * inv * (p.nw != nullptr ? p.nw[p.norm_full ? h * V + c : c] : 1.f));
   }
+}
+
+template <int DQ, int TC, int NC, bool PRE>
+void launch_scan_pre(const LinearAttnArgs& a, int T, const float4* vec, const float* vals, float* oraw, int CH, float* cstate,
+                 float* cdecay, hipStream_t st) {
+  const int cols = (a.V + 8 * NC - 1) / (8 * NC);
+  if (CH <= 0) {
+    hipLaunchKernelGGL((linear_scan_kernel<DQ, TC, NC, SCAN_WHOLE, PRE>), dim3(a.S, a.H, cols), dim3(64), 0, st, a, vec, vals,
+                       oraw, 0, nullptr, nullptr);
+    return;
+  }
+  const int chunks = linear_attn_chunks(T, a.S, CH);
+  hipLaunchKernelGGL((linear_scan_kernel<DQ, TC, NC, SCAN_LOCAL, false>), dim3(chunks, a.H, cols), dim3(64), 0, st, a, vec, vals,
+                     oraw, CH, cstate, cdecay);
+  const int ez = min(64, (a.D * a.V + 255) / 256);
+  hipLaunchKernelGGL(linear_carry_kernel, dim3(a.S, a.H, ez), dim3(256), 0, st, a, CH, cstate, cdecay);
+  hipLaunchKernelGGL((linear_scan_kernel<DQ, TC, NC, SCAN_OUTPUT, PRE>), dim3(chunks, a.H, cols), dim3(64), 0, st, a, vec, vals,
+                     oraw, CH, cstate, cdecay);
 }
 
 template <int DQ, int TC, int NC>
 void launch_scan(const LinearAttnArgs& a, int T, const float4* vec, const float* vals, float* oraw, int CH, float* cstate,
                  float* cdecay, hipStream_t st) {
-  const int cols = (a.V + 8 * NC - 1) / (8 * NC);
-  if (CH <= 0) {
-    hipLaunchKernelGGL((linear_scan_kernel<DQ, TC, NC, SCAN_WHOLE>), dim3(a.S, a.H, cols), dim3(64), 0, st, a, vec, vals,
-                       oraw, 0, nullptr, nullptr);
-    return;
-  }
-  const int chunks = linear_attn_chunks(T, a.S, CH);
-  hipLaunchKernelGGL((linear_scan_kernel<DQ, TC, NC, SCAN_LOCAL>), dim3(chunks, a.H, cols), dim3(64), 0, st, a, vec, vals,
-                     oraw, CH, cstate, cdecay);
-  const int ez = min(64, (a.D * a.V + 255) / 256);
-  hipLaunchKernelGGL(linear_carry_kernel, dim3(a.S, a.H, ez), dim3(256), 0, st, a, CH, cstate, cdecay);
-  hipLaunchKernelGGL((linear_scan_kernel<DQ, TC, NC, SCAN_OUTPUT>), dim3(chunks, a.H, cols), dim3(64), 0, st, a, vec, vals,
-                     oraw, CH, cstate, cdecay);
+  if (a.bonus != nullptr) launch_scan_pre<DQ, TC, NC, true>(a, T, vec, vals, oraw, CH, cstate, cdecay, st);
+  else launch_scan_pre<DQ, TC, NC, false>(a, T, vec, vals, oraw, CH, cstate, cdecay, st);
 }
 
 }  // namespace

@@ -81,7 +81,8 @@ __global__ __launch_bounds__(256) void cast_rows_kernel(const float* __restrict_
 
 // out[t][j] = act(gu[t][j]) * gu[t][n + j] for a stacked [gate; up] projection (bf16), 8 columns per thread
 __global__ __launch_bounds__(256) void glu_rows_kernel(const bf16_t* __restrict__ gu, int64_t ldg, bf16_t* __restrict__ out,
-                                                        int64_t ldo, int n, int act, int64_t total) {
+                                                        int64_t ldo, int n, int act, float limit, float alpha,
+                                                        int64_t total) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= total) return;
   const int per = n / 8;
@@ -92,7 +93,12 @@ __global__ __launch_bounds__(256) void glu_rows_kernel(const bf16_t* __restrict_
   unpack8(ld16(gu + t * ldg + n + j), u);
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    const float x = g[e];
+    float x = g[e];
+    if (act == 2) {  // clamped: min(g, L) * sigmoid(alpha min(g, L)) * (clamp(u, -L, L) + 1)
+      x = fminf(x, limit);
+      g[e] = x * sigm(alpha * x) * (fminf(fmaxf(u[e], -limit), limit) + 1.f);
+      continue;
+    }
     const float a = act == 4 ? 0.5f * x * (1.f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x))) : x * sigm(x);
     g[e] = a * u[e];
   }
@@ -298,6 +304,113 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const int32_t* __restric
   }
 }
 
+// x[t] += mult * y[t] (fp32 sum); with w: h[t] = x[t] / sqrt(mean(x[t]^2) + eps) * w from the new row. One workgroup
+// per token; the row stays in registers between the add and the norm (W <= 256 * RN_MAX), else it is read again.
+constexpr int RN_MAX = 16;
+__global__ __launch_bounds__(256) void residual_norm_kernel(float* __restrict__ x, const void* __restrict__ y, int y_f32,
+                                                             float mult, const float* __restrict__ w, float eps,
+                                                             void* __restrict__ h, int h_f32, int W) {
+  __shared__ float red[16];
+  const int t = blockIdx.x;
+  float* xr = x + (int64_t)t * W;
+  float keep[RN_MAX];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < RN_MAX; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    if (c < W) {
+      const float v = fmaf(mult, ldx(y, (int64_t)t * W + c, y_f32), xr[c]);
+      xr[c] = v;
+      keep[i] = v;
+      ss = fmaf(v, v, ss);
+    }
+  }
+  for (int c = threadIdx.x + 256 * RN_MAX; c < W; c += 256) {
+    const float v = fmaf(mult, ldx(y, (int64_t)t * W + c, y_f32), xr[c]);
+    xr[c] = v;
+    ss = fmaf(v, v, ss);
+  }
+  if (w == nullptr) return;  // (uniform)
+  ss = block_reduce_sum(ss, red);
+  const float inv = 1.f / sqrtf(ss / (float)W + eps);
+#pragma unroll
+  for (int i = 0; i < RN_MAX; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    if (c < W) stx(h, (int64_t)t * W + c, h_f32, keep[i] * inv * w[c]);
+  }
+  for (int c = threadIdx.x + 256 * RN_MAX; c < W; c += 256) stx(h, (int64_t)t * W + c, h_f32, xr[c] * inv * w[c]);
+}
+
+// out[t] = [a[t], b[t]] in out's dtype
+__global__ __launch_bounds__(256) void pair_rows_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                         void* __restrict__ out, int out_f32, int W, int64_t total) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int64_t t = i / (2 * W);
+  const int c = (int)(i % (2 * W));
+  stx(out, i, out_f32, c < W ? a[t * W + c] : b[t * W + c - W]);
+}
+
+// out[s][t] = h[t] + (h'[t] - h[t]) * mu[s], h' = the row before (the slot's kept row for a portion's first token,
+// zeros at position 0). blockIdx.x: token. The slot's row is rewritten by shift_keep_kernel in a launch of its own,
+// after every read of it.
+__global__ __launch_bounds__(256) void shift_mix_kernel(const void* __restrict__ h, int h_f32, const float* __restrict__ last,
+                                                         const float* __restrict__ mu, int n,
+                                                         const int32_t* __restrict__ state_slots,
+                                                         const int32_t* __restrict__ context_lens,
+                                                         const int32_t* __restrict__ query_start, int S,
+                                                         void* __restrict__ out, int64_t plane, int W) {
+  const int t = blockIdx.x;
+  if (t >= query_start[S]) return;
+  int lo = 0, hi = S - 1;  // query_start[s] <= t < query_start[s + 1]
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (query_start[mid] <= t) lo = mid; else hi = mid - 1;
+  }
+  const int s = lo, slot = state_slots[s];
+  if (slot < 0) return;
+  const int t0 = query_start[s];
+  const bool first = t == t0;
+  const bool zero = first && context_lens[s] - (query_start[s + 1] - t0) <= 0;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float x = ldx(h, (int64_t)t * W + c, h_f32);
+    const float p = zero ? 0.f : (first ? last[(int64_t)slot * W + c] : ldx(h, (int64_t)(t - 1) * W + c, h_f32));
+    const float d = p - x;
+    for (int k = 0; k < n; ++k) stx(out, (int64_t)k * plane + (int64_t)t * W + c, h_f32, fmaf(d, mu[(int64_t)k * W + c], x));
+  }
+}
+__global__ __launch_bounds__(256) void shift_keep_kernel(const void* __restrict__ h, int h_f32, float* __restrict__ last,
+                                                          const int32_t* __restrict__ state_slots,
+                                                          const int32_t* __restrict__ query_start, int W) {
+  const int s = blockIdx.x, slot = state_slots[s];
+  const int t0 = query_start[s], t1 = query_start[s + 1];
+  if (slot < 0 || t1 <= t0) return;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) last[(int64_t)slot * W + c] = ldx(h, (int64_t)(t1 - 1) * W + c, h_f32);
+}
+
+// a [T][G][2][rep][V] (two maps' results per head) -> out [T][H][V]: o = a1 - lam a2, o / sqrt(mean(o^2) + eps) * scale,
+// times sigmoid(gate). One wave per (token, head).
+__global__ __launch_bounds__(256) void map_pair_combine_kernel(const void* __restrict__ a, int f32, float lam, float scale,
+                                                                float eps, const void* __restrict__ gate, int64_t ldg,
+                                                                void* __restrict__ out, int H, int G, int V, int T) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (row >= T * H) return;
+  const int t = row / H, hd = row % H, rep = H / G, g = hd / rep, r = hd % rep;
+  const int64_t a1 = (((int64_t)t * G + g) * 2 * rep + r) * V, a2 = a1 + (int64_t)rep * V;
+  float ss = 0.f;
+  for (int c = lane; c < V; c += 64) {
+    const float o = ldx(a, a1 + c, f32) - lam * ldx(a, a2 + c, f32);
+    ss = fmaf(o, o, ss);
+  }
+  ss = wave_reduce_sum(ss);
+  const float inv = scale / sqrtf(ss / (float)V + eps);
+  for (int c = lane; c < V; c += 64) {
+    float o = (ldx(a, a1 + c, f32) - lam * ldx(a, a2 + c, f32)) * inv;
+    if (gate != nullptr) o *= sigm(ldx(gate, (int64_t)t * ldg + (int64_t)hd * V + c, f32));
+    stx(out, ((int64_t)t * H + hd) * V + c, f32, o);
+  }
+}
+
 __global__ __launch_bounds__(256) void moe_combine_kernel(const void* __restrict__ y, const int32_t* __restrict__ pos,
                                                            const float* __restrict__ wts, int W, int top, int y_f32,
                                                            const void* __restrict__ add, void* __restrict__ out,
@@ -321,11 +434,40 @@ void launch_cast_rows(const float* x, void* y, int T, int n, hipStream_t st) {
                      reinterpret_cast<bf16_t*>(y), tot);
 }
 
-void launch_glu_rows(const void* gu, int64_t ldg, void* out, int64_t ldo, int T, int n, int act, hipStream_t st) {
+void launch_glu_rows(const void* gu, int64_t ldg, void* out, int64_t ldo, int T, int n, int act, float limit, float alpha,
+                     hipStream_t st) {
   const int64_t total = (int64_t)T * (n / 8);
   if (total <= 0) return;
   hipLaunchKernelGGL(glu_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
-                     reinterpret_cast<const bf16_t*>(gu), ldg, reinterpret_cast<bf16_t*>(out), ldo, n, act, total);
+                     reinterpret_cast<const bf16_t*>(gu), ldg, reinterpret_cast<bf16_t*>(out), ldo, n, act, limit, alpha, total);
+}
+
+void launch_residual_norm(float* x, const void* y, int y_f32, float mult, const float* w, float eps, void* h, int h_f32,
+                          int T, int W, hipStream_t st) {
+  if (T <= 0 || W <= 0) return;
+  hipLaunchKernelGGL(residual_norm_kernel, dim3(T), dim3(256), 0, st, x, y, y_f32, mult, w, eps, h, h_f32, W);
+}
+
+void launch_pair_rows(const float* a, const float* b, void* out, int out_f32, int T, int W, hipStream_t st) {
+  const int64_t total = (int64_t)T * 2 * W;
+  if (total <= 0) return;
+  hipLaunchKernelGGL(pair_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, a, b, out, out_f32, W, total);
+}
+
+void launch_shift_mix(const void* h, int h_f32, float* last, const float* mu, int n, const int32_t* state_slots,
+                      const int32_t* context_lens, const int32_t* query_start, int S, void* out, int64_t plane, int T, int W,
+                      hipStream_t st) {
+  if (T <= 0 || S <= 0 || W <= 0) return;
+  hipLaunchKernelGGL(shift_mix_kernel, dim3(T), dim3(256), 0, st, h, h_f32, last, mu, n, state_slots, context_lens,
+                     query_start, S, out, plane, W);
+  hipLaunchKernelGGL(shift_keep_kernel, dim3(S), dim3(256), 0, st, h, h_f32, last, state_slots, query_start, W);
+}
+
+void launch_map_pair_combine(const void* a, int f32, float lam, float scale, float eps, const void* gate, int64_t ldg,
+                             void* out, int H, int G, int V, int T, hipStream_t st) {
+  if (T <= 0 || H <= 0) return;
+  hipLaunchKernelGGL(map_pair_combine_kernel, dim3((T * H + 3) / 4), dim3(256), 0, st, a, f32, lam, scale, eps, gate, ldg,
+                     out, H, G, V, T);
 }
 
 void launch_post_norm_add(const PostNormArgs& a, hipStream_t st) {

@@ -43,8 +43,25 @@ void launch_gated_residual(float* x, const void* y1, const void* g1, int64_t ldg
 
 // y = x rounded to the activation dtype (bf16), rows of n
 void launch_cast_rows(const float* x, void* y, int T, int n, hipStream_t st);
-// out[t][j] = act(gu[t][j]) * gu[t][n + j], j < n (bf16 rows, n % 8 == 0, 16-B aligned); act 1 silu, 4 gelu_tanh
-void launch_glu_rows(const void* gu, int64_t ldg, void* out, int64_t ldo, int T, int n, int act, hipStream_t st);
+// out[t][j] = act(gu[t][j]) * gu[t][n + j], j < n (bf16 rows, n % 8 == 0, 16-B aligned); act 1 silu, 4 gelu_tanh,
+// 2 clamped: g' = min(g, limit), g' * sigmoid(alpha g') * (clamp(u, -limit, limit) + 1)
+void launch_glu_rows(const void* gu, int64_t ldg, void* out, int64_t ldo, int T, int n, int act, float limit, float alpha,
+                     hipStream_t st);
+// x[t] += mult * y[t] in fp32 (x [T][W]); with w [W]: h[t] = x[t] * rsqrt(mean(x[t]^2) + eps) * w from the new row
+void launch_residual_norm(float* x, const void* y, int y_f32, float mult, const float* w, float eps, void* h, int h_f32,
+                          int T, int W, hipStream_t st);
+// out[t] = [a[t], b[t]] (fp32 rows of W side by side) in out's dtype
+void launch_pair_rows(const float* a, const float* b, void* out, int out_f32, int T, int W, hipStream_t st);
+// out[k][t] = h[t] + (h'[t] - h[t]) * mu[k] for k < n blend vectors mu [n][W] (plane: stride between out's k planes),
+// h' the row of the token before: h[t - 1] inside a sequence's portion, last[slot] for its first token, zeros at
+// position 0; afterwards last[slot] = the portion's last row (a second launch)
+void launch_shift_mix(const void* h, int h_f32, float* last, const float* mu, int n, const int32_t* state_slots,
+                      const int32_t* context_lens, const int32_t* query_start, int S, void* out, int64_t plane, int T, int W,
+                      hipStream_t st);
+// a [T][G][2][H / G][V]: two maps' attention results per head; out [T][H][V] = (a1 - lam a2) * rsqrt(mean(.^2) + eps) *
+// scale * sigmoid(gate[t][h][:]) (gate null: none)
+void launch_map_pair_combine(const void* a, int f32, float lam, float scale, float eps, const void* gate, int64_t ldg,
+                             void* out, int H, int G, int V, int T, hipStream_t st);
 // out = x + u * rsqrt(mean(u^2) + eps) * w, u = s1 y1 [+ s2 y2] (fp32; out may alias x). With hist
 // ([planes][T][W] fp32, plane stride hist_ps, whose last used plane is out): mix = sum_j coef[j] hist[j].
 // act_out (bf16): a copy of mix, or of out without hist.
@@ -75,10 +92,11 @@ void launch_latent_write(const LatentArgs& a, const void* kv, int64_t ldkv, cons
                          int page, hipStream_t st);
 // qa[t][h][rank:] = rope(q[t][h][dim:]) for q laid out [T][H][dim + rot], qa [T][H][rank + rot]
 void launch_latent_qrope(const LatentArgs& a, const void* q, int H, int dim, void* qa, hipStream_t st);
-// ol[t][h][:rank] = softmax_j(scale * qa[t][h] . cache[j]) . cache[j][:rank] over the causal keys
+// ol[t][h][:rank] = softmax_j(scale * qa[t][h] . cache[j]) . cache[j][:rank] over the keys j with
+// 0 <= position(t) - j < window; sink [H] (null: none): exp(sink[h]) is added to the softmax denominator
 void launch_latent_attn(const LatentArgs& a, const void* qa, int H, float scale, const int32_t* block_tables,
                         int max_blocks, int page, const int32_t* context_lens, const int32_t* query_start, int S,
-                        void* ol, const void* cache_t, int num_pages, hipStream_t st);
+                        void* ol, const void* cache_t, int num_pages, int window, const float* sink, hipStream_t st);
 
 struct DeltaArgs {
   const void* r = nullptr; const void* k = nullptr; const void* v = nullptr; const void* g = nullptr;
@@ -98,6 +116,9 @@ void launch_delta_rule(const DeltaArgs& a, int T, float* scratch, hipStream_t st
 // Sliding-window attention over paged key / value caches with optional pooled blocks (window_attn.hip).
 struct WindowArgs {
   int H = 0, G = 0, D = 0, V = 0;       // query heads, key/value heads, key size, value size
+  int GV = 0;                           // value heads (divides G): key head g reads value head g / (G / GV)
+  float softcap = 0.f;                  // c > 0: the scaled score s becomes c tanh(s / c) (not with a distance term)
+  float cap_in = 0.f, cap_out = 0.f;    // (set by launch_window_attn: 2 / c and c log2 e)
   int page = 0, npool = 0;              // tokens per page; pooled rows per page (0: no pooled caches)
   int rot_dims = 0, window = 0, pool = 0;
   int f32 = 0, T = 0, S = 0, max_blocks = 0;
@@ -116,7 +137,7 @@ struct WindowArgs {
   const int32_t* positions = nullptr;   // [T]
   const int32_t* slots = nullptr;       // [T] page * tokens-per-page + offset of each token (-1: padding)
   const int32_t* block_tables = nullptr; const int32_t* context_lens = nullptr; const int32_t* query_start = nullptr;
-  void* kc = nullptr; void* vc = nullptr;  // [pages][G][page][D | V]
+  void* kc = nullptr; void* vc = nullptr;  // [pages][G][page][D], [pages][GV][page][V]
   void* kp = nullptr; void* vp = nullptr;  // [pages][G][npool][D | V]
 };
 size_t window_attn_lds_bytes(const WindowArgs& a, int heads_per_block);
@@ -128,10 +149,11 @@ size_t window_attn_part_floats(int T, int S, int H, int G, int D, int V, int par
 bool window_attn_fits(const WindowArgs& a);   // sizes the kernels' LDS and register budgets take
 // q / k norm (qw, kw null: none; norm_all: one norm over the whole projection) + rotation + paged stores; q_out [T][H * D];
 // the query of head h at position p is multiplied by q_head_scale[h] (null: 1) * (1 + q_temp_coef ln(floor((p + 1) / q_temp_every) + 1));
-// vt: optional second, transposed bf16 copy of the values [pages][G][V][page]
+// vt: optional second, transposed bf16 copy of the values [pages][GV][V][page]; rot_half: entry i is paired with
+// entry i + rot_dims / 2 instead of 2i with 2i + 1
 void launch_window_write(const WindowArgs& a, const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v,
                          int64_t ldv, const float* qw, const float* kw, float eps, int norm_all, void* q_out, void* vt,
-                         const float* q_head_scale, float q_temp_coef, int q_temp_every, hipStream_t st);
+                         const float* q_head_scale, float q_temp_coef, int q_temp_every, int rot_half, hipStream_t st);
 // pooled rows of the blocks this step's tokens complete
 void launch_window_pool(const WindowArgs& a, hipStream_t st);
 // out[t][h][:V] = softmax over (pooled blocks before the window, window tokens [, sink]) of scale q . key, times values
@@ -159,6 +181,9 @@ struct LinearAttnArgs {
   void* out = nullptr; int64_t ldo = 0;
   int S = 0, H = 0, D = 0, V = 0, f32 = 0;
   int cols_per_lane = 0;                        // value columns per lane of the scan: 0 = by the launch's size, 1, or > 1 (wide)
+  int decay_exp = 0;                            // a = exp(-exp(z)) instead of sigmoid(z)^(1 / tau)
+  const float* bonus = nullptr;                 // [H * D]: read the state before its update, o_t = (S + diag(bonus) k v^T)^T q
+  int norm_full = 0;                            // per-head norm with a weight [H * V] (one entry per output channel)
 };
 // tokens per chunk a step of T rows over S sequences is scanned in (0: every sequence in one pass), the
 // chunks such a step has at most, and the scratch floats it needs

@@ -34,6 +34,9 @@
 //               n = i - j alone, -r1[h] ln(1 + r2[h] n) or a table entry tab[h][min(n, last)]; the MFMA kernels
 //               compute it in log2 units beside the mask (the table of a workgroup's heads staged in LDS when
 //               it fits). An output gate multiplies the normalised result by sigmoid(gate) in the epilogue.
+// Softcap c > 0 (not with a distance term): the scaled score s becomes c tanh(s / c) (CAP instantiations of the MFMA
+//               kernels). The value caches may have fewer heads (GV) than the key cache: key head g reads value head
+//               g / (G / GV), which is how two score maps of one head share their values.
 // Every row of every kernel depends only on its own sequence's cache rows, in an order fixed by the
 // position, so results do not depend on how a prompt is cut or what else is in the batch.
 #include "common.h"
@@ -65,9 +68,9 @@ __global__ __launch_bounds__(256) void window_write_kernel(WindowArgs a, const v
                                                             const float* __restrict__ qw, const float* __restrict__ kw,
                                                             float eps, int norm_all, void* __restrict__ q_out,
                                                             bf16_t* __restrict__ vt, const float* __restrict__ q_head_scale,
-                                                            float q_temp_coef, int q_temp_every) {
+                                                            float q_temp_coef, int q_temp_every, int rot_half) {
   extern __shared__ float lds[];
-  const int H = a.H, G = a.G, D = a.D, V = a.V;
+  const int H = a.H, G = a.G, D = a.D, V = a.V, GV = a.GV;
   float* xs = lds;                    // [(H + G) * D] q heads then k heads
   float* inv = xs + (H + G) * D;      // [H + G]
   const int t = blockIdx.x;
@@ -110,12 +113,14 @@ __global__ __launch_bounds__(256) void window_write_kernel(WindowArgs a, const v
     const int wo = norm_all ? (isq ? h : h - H) * D : 0;
     const float sc = w != nullptr ? inv[h] : 1.f;
     float o;
-    if (i < a.rot_dims) {
-      const int i0 = i & ~1, i1 = i | 1;
+    if (i < a.rot_dims) {  // the pair (i0, i1) = (2j, 2j + 1), or (j, j + rot_dims / 2) with rot_half
+      const int hr = a.rot_dims >> 1;
+      const int j = rot_half ? (i < hr ? i : i - hr) : (i >> 1);
+      const int i0 = rot_half ? j : (i & ~1), i1 = rot_half ? j + hr : (i | 1);
       const float x0 = xs[h * D + i0] * sc * (w ? w[wo + i0] : 1.f), x1 = xs[h * D + i1] * sc * (w ? w[wo + i1] : 1.f);
-      const float ang = pos * a.inv_freq[i >> 1];
+      const float ang = pos * a.inv_freq[j];
       const float cs = cosf(ang), sn = sinf(ang);
-      o = (i & 1) ? (x1 * cs + x0 * sn) : (x0 * cs - x1 * sn);
+      o = (i == i1) ? (x1 * cs + x0 * sn) : (x0 * cs - x1 * sn);
     } else {
       o = xs[h * D + i] * sc * (w ? w[wo + i] : 1.f);
     }
@@ -123,7 +128,7 @@ __global__ __launch_bounds__(256) void window_write_kernel(WindowArgs a, const v
     else stx(a.kc, ((pg * G + (h - H)) * page + off) * D + i, a.f32, o);
   }
   const int vrot = a.v_freq != nullptr ? 2 * (V / 2) : 0;
-  for (int e = tid; e < G * V; e += 256) {
+  for (int e = tid; e < GV * V; e += 256) {
     const int g = e / V, i = e % V;
     float o;
     if (i < vrot) {
@@ -134,8 +139,8 @@ __global__ __launch_bounds__(256) void window_write_kernel(WindowArgs a, const v
     } else {
       o = ldx(v, (int64_t)t * ldv + e, a.f32);
     }
-    stx(a.vc, ((pg * G + g) * page + off) * V + i, a.f32, o);
-    if (vt != nullptr) vt[((pg * G + g) * V + i) * page + off] = f2bf(o);  // [page][G][column][key in page]
+    stx(a.vc, ((pg * GV + g) * page + off) * V + i, a.f32, o);
+    if (vt != nullptr) vt[((pg * GV + g) * V + i) * page + off] = f2bf(o);  // [page][GV][column][key in page]
   }
 }
 
@@ -215,6 +220,7 @@ __global__ __launch_bounds__(256) void window_attn_kernel(WindowArgs a, const vo
   const int s = seq_of_token(a.query_start, a.S, t);
   const int pos = a.context_lens[s] - (a.query_start[s + 1] - t);  // position of token t
   const int g = blockIdx.y;
+  const int gv = g / (G / a.GV);           // the value head of key head g
   const int rep = a.H / G;
   const int r0 = blockIdx.z * HC;          // first query head of the group handled here
   const int nh = min(HC, rep - r0);
@@ -249,7 +255,8 @@ __global__ __launch_bounds__(256) void window_attn_kernel(WindowArgs a, const vo
           val = ldx(isk ? a.kp : a.vp, row * w + ci, a.f32);
         } else {
           const int j = lo + kj - nb;
-          const int64_t row = ((int64_t)bt[j / page] * G + g) * page + j % page;
+          const int64_t row = isk ? ((int64_t)bt[j / page] * G + g) * page + j % page
+                                  : ((int64_t)bt[j / page] * a.GV + gv) * page + j % page;
           val = ldx(isk ? a.kc : a.vc, row * w + ci, a.f32);
         }
       }
@@ -274,7 +281,9 @@ __global__ __launch_bounds__(256) void window_attn_kernel(WindowArgs a, const vo
         bias = a.bias_kind == 1 ? -a.bias_a[h0 + h] * logf(1.f + a.bias_b[h0 + h] * (float)n)
                                 : a.bias_a[(int64_t)(h0 + h) * a.bias_n + min(n, a.bias_n - 1)];
       }
-      if (on && half == 0) sc[h * KT + jj] = (j0 + jj < nkeys) ? d * scale + bias : -INFINITY;
+      float sv = d * scale;
+      if (a.softcap > 0.f) sv = a.softcap * tanhf(sv / a.softcap);
+      if (on && half == 0) sc[h * KT + jj] = (j0 + jj < nkeys) ? sv + bias : -INFINITY;
     }
     __syncthreads();
     if (tid < nh) {
@@ -419,7 +428,16 @@ __device__ __forceinline__ float gate_of(const bf16_t* grow, int col) { return 1
 // output column (never stored) makes the value irrelevant, and cached values are always finite.
 constexpr int LG = 4;
 // NW: waves of a workgroup, which share out the key tiles of its 16 rows
-template <int NCT, int NQF, int NW, int BIAS>
+// the score of one key in log2 units: the scaled score, softcapped (CAP) or with its distance term (BIAS) added
+template <bool CAP>
+__device__ __forceinline__ float score_log2(const WindowArgs& a, float s, float scale_log2e, float bias) {
+  if (!CAP) return fmaf(s, scale_log2e, bias);
+  // cap tanh(x / cap) log2e with x / cap = s scale / cap; tanh(y) = 1 - 2 / (e^(2y) + 1), exact at both ends
+  const float e = exp2f(s * scale_log2e * a.cap_in);   // cap_in = 2 / cap
+  return a.cap_out * (1.f - 2.f / (e + 1.f));          // cap_out = cap log2e
+}
+
+template <int NCT, int NQF, int NW, int BIAS, bool CAP>
 __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a, const bf16_t* __restrict__ q,
                                                                 float scale_log2e, const bf16_t* __restrict__ vt,
                                                                 int num_pages, bf16_t* __restrict__ out) {
@@ -428,6 +446,7 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
   __shared__ float mrg_m[NW][16], mrg_l[NW][16];
   __shared__ float mrg_o[16][16 * NCT];  // the merged weighted values of the 16 rows
   const int D = a.D, V = a.V, G = a.G, H = a.H, rep = H / G, g = blockIdx.y, P = a.pool;
+  const int GV = a.GV, gv = g / (G / GV);  // value heads; the value head of key head g
   int s = -1, tile = 0, base = 0;
   for (int i = 0; i < a.S; ++i) {  // (sequence, 16-row tile) of this workgroup
     const int nt = ((a.query_start[i + 1] - a.query_start[i]) * rep + 15) / 16;
@@ -540,8 +559,8 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
     for (int i = 0; i < 4; ++i) {
       const bool vis0 = pooled ? c0 < nbv[i] : (c0 >= lo[i] && c0 <= hi[i]);
       const bool vis1 = pooled ? c1 < nbv[i] : (c1 >= lo[i] && c1 <= hi[i]);
-      const float v0 = vis0 ? fmaf(s0[i], scale_log2e, BIAS ? bt0[i] : 0.f) : -INFINITY;
-      const float v1 = vis1 ? fmaf(s1[i], scale_log2e, BIAS ? bt1[i] : 0.f) : -INFINITY;
+      const float v0 = vis0 ? score_log2<CAP>(a, s0[i], scale_log2e, BIAS ? bt0[i] : 0.f) : -INFINITY;
+      const float v1 = vis1 ? score_log2<CAP>(a, s1[i], scale_log2e, BIAS ? bt1[i] : 0.f) : -INFINITY;
       const float mnew = fmaxf(m[i], group16_max(fmaxf(v0, v1)));
       const float ms = (mnew == -INFINITY) ? 0.f : mnew;  // a row that has seen no key yet
       al[i] = exp2f(m[i] - ms);
@@ -559,7 +578,7 @@ __global__ __launch_bounds__(64 * NW) void window_attn_mfma_kernel(WindowArgs a,
     const bf16x8 pf = as_bf16x8(*reinterpret_cast<const uint4*>(&pl[wv][lr][8 * lg]));
     if (!pooled) {
       const int pgs = (lg >> 1) ? pg1 : pg0;
-      const bf16_t* tp = vt + ((int64_t)pgs * G + g) * V * 16 + 8 * (lg & 1);
+      const bf16_t* tp = vt + ((int64_t)pgs * GV + gv) * V * 16 + 8 * (lg & 1);
 #pragma unroll
       for (int cb = 0; cb < NCT; cb += 2 * LG) {
         if (cb < nct) {  // wave-uniform
@@ -734,7 +753,7 @@ __global__ __launch_bounds__(256) void window_attn_merge_kernel(WindowArgs a, in
 // and transposed values are brought into LDS once per workgroup (two buffers: tile t + 1 is asked for before
 // tile t is computed, written after it, one barrier per tile), and every wave takes its fragments from there.
 // Pooled tiles come first and are read straight from the pooled caches by each wave, as in the kernel above.
-template <int NCT, int NQF, int BIAS>
+template <int NCT, int NQF, int BIAS, bool CAP>
 __global__ __launch_bounds__(256) void window_attn_tiled_kernel(WindowArgs a, const bf16_t* __restrict__ q,
                                                                  float scale_log2e, const bf16_t* __restrict__ vt,
                                                                  int num_pages, bf16_t* __restrict__ out) {
@@ -746,6 +765,7 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(WindowArgs a, co
   __shared__ __attribute__((aligned(16))) bf16_t vl[2][16 * NCT][VP];
   __shared__ __attribute__((aligned(16))) bf16_t pl[4][16][40];
   const int D = a.D, V = a.V, G = a.G, H = a.H, rep = H / G, g = blockIdx.y, P = a.pool;
+  const int GV = a.GV, gv = g / (G / GV);  // value heads; the value head of key head g
   int s = -1, tile = 0, base = 0;
   for (int i = 0; i < a.S; ++i) {  // (sequence, 64-row tile) of this workgroup
     const int nt = ((a.query_start[i + 1] - a.query_start[i]) * rep + 63) / 64;
@@ -823,8 +843,8 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(WindowArgs a, co
     for (int i = 0; i < 4; ++i) {
       const bool vis0 = pooled ? c0 < nbv[i] : (c0 >= lo[i] && c0 <= hi[i]);
       const bool vis1 = pooled ? c1 < nbv[i] : (c1 >= lo[i] && c1 <= hi[i]);
-      const float v0 = vis0 ? fmaf(s0[i], scale_log2e, BIAS ? bt0[i] : 0.f) : -INFINITY;
-      const float v1 = vis1 ? fmaf(s1[i], scale_log2e, BIAS ? bt1[i] : 0.f) : -INFINITY;
+      const float v0 = vis0 ? score_log2<CAP>(a, s0[i], scale_log2e, BIAS ? bt0[i] : 0.f) : -INFINITY;
+      const float v1 = vis1 ? score_log2<CAP>(a, s1[i], scale_log2e, BIAS ? bt1[i] : 0.f) : -INFINITY;
       const float mnew = fmaxf(m[i], group16_max(fmaxf(v0, v1)));
       const float ms = (mnew == -INFINITY) ? 0.f : mnew;
       al[i] = exp2f(m[i] - ms);
@@ -898,7 +918,7 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(WindowArgs a, co
       const int c = tid + 256 * u;
       const int col = c >> 2, half = (c >> 1) & 1, sub = c & 1;
       const int pg = half ? pg1 : pg0;
-      vr[u] = col < V ? ld16(vt + (((int64_t)pg * G + g) * V + col) * 16 + 8 * sub) : make_uint4(0, 0, 0, 0);
+      vr[u] = col < V ? ld16(vt + (((int64_t)pg * GV + gv) * V + col) * 16 + 8 * sub) : make_uint4(0, 0, 0, 0);
     }
   };
   auto stage = [&](int buf) {
@@ -970,7 +990,7 @@ __global__ __launch_bounds__(256) void window_attn_tiled_kernel(WindowArgs a, co
   }
 }
 
-template <int NCT, int NQF, int BIAS>
+template <int NCT, int NQF, int BIAS, bool CAP>
 void launch_window_mfma(const WindowArgs& a, const void* q, float scale, const void* vt, int num_pages, void* out,
                         hipStream_t st) {
   const int rep = a.H / a.G;
@@ -985,14 +1005,14 @@ void launch_window_mfma(const WindowArgs& a, const void* q, float scale, const v
   // 16 rows per workgroup with the key tiles shared out over four waves)
   if ((int64_t)a.T * rep <= 16 * (int64_t)a.S) {
     const int parts = a.parts > 1 ? a.parts : 1;
-    hipLaunchKernelGGL((window_attn_mfma_kernel<NCT, NQF, 8, BIAS>), dim3(blocks, a.G, parts), dim3(512), dyn, st, a, qp, sl, vp,
+    hipLaunchKernelGGL((window_attn_mfma_kernel<NCT, NQF, 8, BIAS, CAP>), dim3(blocks, a.G, parts), dim3(512), dyn, st, a, qp, sl, vp,
                        num_pages, op);
     if (parts > 1) hipLaunchKernelGGL(window_attn_merge_kernel, dim3(blocks, a.G, 4), dim3(256), 0, st, a, 16 * NCT, op);
   }
   else if (a.prefill_kernel == 1 || NCT > 8)
-    hipLaunchKernelGGL((window_attn_mfma_kernel<NCT, NQF, 4, BIAS>), dim3(blocks, a.G), dim3(256), dyn, st, a, qp, sl, vp, num_pages, op);
+    hipLaunchKernelGGL((window_attn_mfma_kernel<NCT, NQF, 4, BIAS, CAP>), dim3(blocks, a.G), dim3(256), dyn, st, a, qp, sl, vp, num_pages, op);
   else
-    hipLaunchKernelGGL((window_attn_tiled_kernel<NCT, NQF, BIAS>), dim3((a.T * rep + 63) / 64 + a.S, a.G), dim3(256), dyn, st, a, qp, sl,
+    hipLaunchKernelGGL((window_attn_tiled_kernel<NCT, NQF, BIAS, CAP>), dim3((a.T * rep + 63) / 64 + a.S, a.G), dim3(256), dyn, st, a, qp, sl,
                        vp, num_pages, op);
 }
 
@@ -1000,13 +1020,13 @@ void launch_window_mfma(const WindowArgs& a, const void* q, float scale, const v
 int window_attn_nct(int D, int V);
 namespace {
 
-template <int BIAS>
+template <int BIAS, bool CAP>
 void launch_window_mfma_sized(const WindowArgs& a, const void* q, float scale, const void* vt, int num_pages, void* out,
                               hipStream_t st) {
   const int nct = window_attn_nct(a.D, a.V);  // (the scratch of a split launch is sized by the same rule)
-  if (nct == 4) launch_window_mfma<4, 2, BIAS>(a, q, scale, vt, num_pages, out, st);
-  else if (nct == 8) launch_window_mfma<8, 4, BIAS>(a, q, scale, vt, num_pages, out, st);
-  else launch_window_mfma<16, 8, BIAS>(a, q, scale, vt, num_pages, out, st);
+  if (nct == 4) launch_window_mfma<4, 2, BIAS, CAP>(a, q, scale, vt, num_pages, out, st);
+  else if (nct == 8) launch_window_mfma<8, 4, BIAS, CAP>(a, q, scale, vt, num_pages, out, st);
+  else launch_window_mfma<16, 8, BIAS, CAP>(a, q, scale, vt, num_pages, out, st);
 }
 
 int heads_per_block(const WindowArgs& a) {
@@ -1047,11 +1067,11 @@ bool window_attn_fits(const WindowArgs& a) {
 
 void launch_window_write(const WindowArgs& a, const void* q, int64_t ldq, const void* k, int64_t ldk, const void* v,
                          int64_t ldv, const float* qw, const float* kw, float eps, int norm_all, void* q_out, void* vt,
-                         const float* q_head_scale, float q_temp_coef, int q_temp_every, hipStream_t st) {
+                         const float* q_head_scale, float q_temp_coef, int q_temp_every, int rot_half, hipStream_t st) {
   if (a.T <= 0) return;
   const size_t lds = (size_t)((a.H + a.G) * a.D + a.H + a.G) * sizeof(float);
   hipLaunchKernelGGL(window_write_kernel, dim3(a.T), dim3(256), lds, st, a, q, ldq, k, ldk, v, ldv, qw, kw, eps, norm_all,
-                     q_out, reinterpret_cast<bf16_t*>(vt), q_head_scale, q_temp_coef, q_temp_every);
+                     q_out, reinterpret_cast<bf16_t*>(vt), q_head_scale, q_temp_coef, q_temp_every, rot_half);
 }
 
 void launch_window_pool(const WindowArgs& a, hipStream_t st) {
@@ -1061,12 +1081,15 @@ void launch_window_pool(const WindowArgs& a, hipStream_t st) {
   else hipLaunchKernelGGL(window_pool_kernel<bf16_t>, grid, dim3(256), 0, st, a);
 }
 
-void launch_window_attn(const WindowArgs& a, const void* q, float scale, void* out, const void* vt, int num_pages,
+void launch_window_attn(const WindowArgs& a0, const void* q, float scale, void* out, const void* vt, int num_pages,
                         hipStream_t st) {
-  if (a.T <= 0 || a.S <= 0) return;
+  if (a0.T <= 0 || a0.S <= 0) return;
+  WindowArgs a = a0;
+  if (a.softcap > 0.f) { a.cap_in = 2.f / a.softcap; a.cap_out = a.softcap * 1.4426950408889634f; }
   if (!a.f32 && vt != nullptr && a.page == 16 && a.D % 8 == 0 && a.D >= 8 && a.D <= 256 && a.V <= 256) {
-    if (a.bias_kind != 0) launch_window_mfma_sized<1>(a, q, scale, vt, num_pages, out, st);
-    else launch_window_mfma_sized<0>(a, q, scale, vt, num_pages, out, st);
+    if (a.bias_kind != 0) launch_window_mfma_sized<1, false>(a, q, scale, vt, num_pages, out, st);
+    else if (a.softcap > 0.f) launch_window_mfma_sized<0, true>(a, q, scale, vt, num_pages, out, st);
+    else launch_window_mfma_sized<0, false>(a, q, scale, vt, num_pages, out, st);
     return;
   }
   const int HC = heads_per_block(a);

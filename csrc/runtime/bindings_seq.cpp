@@ -189,8 +189,9 @@ void latent_qrope(const Tensor& q, const Tensor& positions, const Tensor& inv_fr
 
 void latent_attn(const Tensor& qa, const Tensor& cache, const Tensor& block_tables, const Tensor& context_lens,
                  const Tensor& query_start, Tensor& ol, double scale, int64_t H, int64_t rank, int64_t rot,
-                 const OptT& cache_t) {
+                 const OptT& cache_t, int64_t window, const OptT& sink) {
   const int f = act_f32(qa, "qa");
+  TORCH_CHECK(window >= 1 && window <= (1 << 30), "latent_attn: window 1 .. 2^30");
   const int64_t E = rank + rot;
   TORCH_CHECK(qa.is_contiguous() && qa.numel() % (H * E) == 0, "latent_attn: qa [T, H, rank + rot]");
   const int64_t T = qa.numel() / (H * E);
@@ -213,7 +214,8 @@ void latent_attn(const Tensor& qa, const Tensor& cache, const Tensor& block_tabl
   }
   c10::DeviceGuard guard(qa.device());
   vgate::launch_latent_attn(a, qa.data_ptr(), (int)H, (float)scale, bt, (int)block_tables.size(1), (int)cache.size(1),
-                            cl, qs, (int)S, ol.data_ptr(), ct, (int)cache.size(0), cur_stream());
+                            cl, qs, (int)S, ol.data_ptr(), ct, (int)cache.size(0), (int)window, f32p(sink, "sink", H),
+                            cur_stream());
 }
 
 void delta_rule(const Tensor& r, const Tensor& k, const Tensor& v, const Tensor& g, const Tensor& a, const Tensor& wl,
@@ -261,7 +263,7 @@ void cast_rows(const Tensor& x, Tensor& y) {
   vgate::launch_cast_rows(x.data_ptr<float>(), y.data_ptr(), (int)y.size(0), (int)y.size(1), cur_stream());
 }
 
-void glu_rows(const Tensor& gu, Tensor& out, int64_t act) {
+void glu_rows(const Tensor& gu, Tensor& out, int64_t act, double limit, double alpha) {
   TORCH_CHECK(gu.is_cuda() && gu.scalar_type() == torch::kBFloat16 && gu.dim() == 2 && gu.stride(1) == 1, "glu_rows: gu bf16 [T, 2 n]");
   TORCH_CHECK(out.is_cuda() && out.scalar_type() == torch::kBFloat16 && out.dim() == 2 && out.stride(1) == 1 &&
               out.size(0) <= gu.size(0) && gu.size(1) == 2 * out.size(1), "glu_rows: out bf16 [<= T, n]");
@@ -269,10 +271,81 @@ void glu_rows(const Tensor& gu, Tensor& out, int64_t act) {
   TORCH_CHECK(n % 8 == 0 && gu.stride(0) % 8 == 0 && out.stride(0) % 8 == 0 &&
               (reinterpret_cast<uintptr_t>(gu.data_ptr()) & 15) == 0 && (reinterpret_cast<uintptr_t>(out.data_ptr()) & 15) == 0,
               "glu_rows: rows of whole 16-B pieces");
-  TORCH_CHECK(act == 1 || act == 4, "glu_rows: act 1 (silu) or 4 (gelu_tanh)");
+  TORCH_CHECK(act == 1 || act == 2 || act == 4, "glu_rows: act 1 (silu), 2 (clamped) or 4 (gelu_tanh)");
   c10::DeviceGuard guard(gu.device());
   vgate::launch_glu_rows(gu.data_ptr(), gu.stride(0), out.data_ptr(), out.stride(0), (int)out.size(0), (int)n, (int)act,
-                         cur_stream());
+                         (float)limit, (float)alpha, cur_stream());
+}
+
+void residual_norm(Tensor& x, const Tensor& y, double mult, const OptT& w, double eps, const OptT& h_out) {
+  TORCH_CHECK(x.is_cuda() && x.scalar_type() == torch::kFloat32 && x.is_contiguous() && x.dim() == 2, "residual_norm: x fp32 [T, W]");
+  const int yf = act_f32(y, "y");
+  const int64_t T = y.size(0), W = x.size(1);
+  TORCH_CHECK(y.dim() == 2 && y.is_contiguous() && y.size(1) == W && T <= x.size(0), "residual_norm: y [<= T, W]");
+  const float* wp = f32p(w, "w", W);
+  void* hp = nullptr;
+  int hf = 0;
+  TORCH_CHECK(has(w) == has(h_out), "residual_norm: the norm weight and its output come together");
+  if (has(h_out)) {
+    hf = act_f32(*h_out, "h_out");
+    TORCH_CHECK(h_out->dim() == 2 && h_out->is_contiguous() && h_out->size(1) == W && h_out->size(0) >= T, "residual_norm: h_out [T, W]");
+    hp = h_out->data_ptr();
+  }
+  c10::DeviceGuard guard(x.device());
+  vgate::launch_residual_norm(x.data_ptr<float>(), y.data_ptr(), yf, (float)mult, wp, (float)eps, hp, hf, (int)T, (int)W,
+                              cur_stream());
+}
+
+void pair_rows(const Tensor& a, const Tensor& b, Tensor& out) {
+  const int of = act_f32(out, "out");
+  TORCH_CHECK(out.dim() == 2 && out.is_contiguous() && out.size(1) % 2 == 0, "pair_rows: out [T, 2 W]");
+  const int64_t T = out.size(0), W = out.size(1) / 2;
+  for (const Tensor* t : {&a, &b})
+    TORCH_CHECK(t->is_cuda() && t->scalar_type() == torch::kFloat32 && t->is_contiguous() && t->dim() == 2 && t->size(0) >= T &&
+                t->size(1) == W, "pair_rows: fp32 [>= T, W] inputs");
+  c10::DeviceGuard guard(out.device());
+  vgate::launch_pair_rows(a.data_ptr<float>(), b.data_ptr<float>(), out.data_ptr(), of, (int)T, (int)W, cur_stream());
+}
+
+void shift_mix(const Tensor& h, Tensor& last, const Tensor& mu, const Tensor& state_slots, const Tensor& context_lens,
+               const Tensor& query_start, Tensor& out) {
+  const int hf = act_f32(h, "h");
+  TORCH_CHECK(h.dim() == 2 && h.is_contiguous(), "shift_mix: h [T, W]");
+  const int64_t T = h.size(0), W = h.size(1);
+  TORCH_CHECK(last.is_cuda() && last.scalar_type() == torch::kFloat32 && last.is_contiguous() && last.dim() == 2 &&
+              last.size(1) == W, "shift_mix: last fp32 [slots, W]");
+  TORCH_CHECK(mu.dim() == 2 && mu.size(1) == W, "shift_mix: mu [n, W]");
+  OptT mo(mu);
+  const float* mp = f32p(mo, "mu", -1);
+  const int64_t n = mu.size(0);
+  TORCH_CHECK(act_f32(out, "out") == hf && out.dim() == 3 && out.is_contiguous() && out.size(0) == n && out.size(1) == T &&
+              out.size(2) == W, "shift_mix: out [n, T, W] of h's dtype");
+  const int64_t S = state_slots.numel();
+  const int32_t* sp = i32p(state_slots, "state_slots", S);  // values < slots (or -1): set by the slot manager
+  const int32_t* cl = i32p(context_lens, "context_lens", S);
+  const int32_t* qs = i32p(query_start, "query_start", S + 1);
+  c10::DeviceGuard guard(h.device());
+  vgate::launch_shift_mix(h.data_ptr(), hf, last.data_ptr<float>(), mp, (int)n, sp, cl, qs, (int)S, out.data_ptr(),
+                          T * W, (int)T, (int)W, cur_stream());
+}
+
+void map_pair_combine(const Tensor& a, double lam, double out_scale, double eps, const OptT& gate, Tensor& out, int64_t H,
+                      int64_t G, int64_t V) {
+  const int f = act_f32(a, "a");
+  TORCH_CHECK(G >= 1 && H % G == 0 && V >= 1, "map_pair_combine: heads a multiple of key/value heads");
+  TORCH_CHECK(out.dim() == 2 && out.is_contiguous() && act_f32(out, "out") == f && out.size(1) == H * V, "map_pair_combine: out [T, H V]");
+  const int64_t T = out.size(0);
+  TORCH_CHECK(a.dim() == 2 && a.is_contiguous() && a.size(0) >= T && a.size(1) == 2 * H * V, "map_pair_combine: a [T, 2 H V]");
+  const void* gp = nullptr;
+  int64_t ldg = 0;
+  if (has(gate)) {
+    TORCH_CHECK(act_f32(*gate, "gate") == f && gate->dim() == 2 && gate->size(0) >= T && gate->size(1) == H * V,
+                "map_pair_combine: gate [T, H V] of a's dtype");
+    gp = gate->data_ptr(); ldg = gate->stride(0);
+  }
+  c10::DeviceGuard guard(a.device());
+  vgate::launch_map_pair_combine(a.data_ptr(), f, (float)lam, (float)out_scale, (float)eps, gp, ldg, out.data_ptr(), (int)H,
+                                 (int)G, (int)V, (int)T, cur_stream());
 }
 
 void post_norm_add(const Tensor& x, const Tensor& y1, const Tensor& w, double eps, Tensor& out, double s1, const OptT& y2,
@@ -320,9 +393,11 @@ vgate::WindowArgs window_common(const Tensor& kc, const Tensor& vc, const OptT& 
   vgate::WindowArgs a;
   a.f32 = act_f32(kc, "kc");
   TORCH_CHECK(kc.dim() == 4 && vc.dim() == 4 && kc.is_contiguous() && vc.is_contiguous() && act_f32(vc, "vc") == a.f32 &&
-              kc.size(0) == vc.size(0) && kc.size(1) == vc.size(1) && kc.size(2) == vc.size(2),
-              "window: kc [pages, G, page, D], vc [pages, G, page, V] of one dtype");
+              kc.size(0) == vc.size(0) && vc.size(1) >= 1 && kc.size(1) % vc.size(1) == 0 && kc.size(2) == vc.size(2),
+              "window: kc [pages, G, page, D], vc [pages, GV, page, V] of one dtype, GV dividing G");
   a.G = (int)kc.size(1); a.page = (int)kc.size(2); a.D = (int)kc.size(3); a.V = (int)vc.size(3); a.H = (int)H;
+  a.GV = (int)vc.size(1);
+  TORCH_CHECK(pool == 0 || a.GV == a.G, "window: pooled blocks need one value head per key head");
   TORCH_CHECK(a.G >= 1 && H >= a.G && H % a.G == 0 && H + a.G <= 256, "window: heads a multiple of kv heads, at most 256 together");
   a.kc = kc.data_ptr(); a.vc = vc.data_ptr();
   a.pool = (int)pool;
@@ -352,14 +427,15 @@ void* window_vt(const OptT& vt, const Tensor& vc) {
 void window_write(const Tensor& q, const Tensor& k, const Tensor& v, const OptT& qw, const OptT& kw, double eps,
                   bool norm_all, const Tensor& positions, const Tensor& slots, const Tensor& inv_freq, int64_t rot_dims,
                   const OptT& v_freq, Tensor& kc, Tensor& vc, Tensor& q_out, int64_t H, int64_t G, const OptT& vt,
-                  const OptT& q_head_scale, double q_temp_coef, int64_t q_temp_every) {
+                  const OptT& q_head_scale, double q_temp_coef, int64_t q_temp_every, bool rot_half) {
   auto a = window_common(kc, vc, c10::nullopt, c10::nullopt, H, 0);
   TORCH_CHECK(q_temp_every >= 1, "window_write: q_temp_every >= 1");
   TORCH_CHECK(G == a.G, "window_write: kv heads");
   const int64_t T = q.size(0);
   TORCH_CHECK(act_f32(q, "q") == a.f32 && act_f32(k, "k") == a.f32 && act_f32(v, "v") == a.f32 && q.dim() == 2 &&
               k.dim() == 2 && v.dim() == 2 && k.size(0) == T && v.size(0) == T && q.size(1) == H * a.D &&
-              k.size(1) == G * a.D && v.size(1) == G * a.V, "window_write: q [T, H D], k [T, G D], v [T, G V] of the caches' dtype");
+              k.size(1) == G * a.D && v.size(1) == (int64_t)a.GV * a.V,
+              "window_write: q [T, H D], k [T, G D], v [T, GV V] of the caches' dtype");
   TORCH_CHECK(act_f32(q_out, "q_out") == a.f32 && q_out.is_contiguous() && q_out.dim() == 2 && q_out.size(0) == T &&
               q_out.size(1) == H * a.D, "window_write: q_out [T, H D]");
   TORCH_CHECK(rot_dims >= 0 && rot_dims <= a.D && rot_dims % 2 == 0, "window_write: rot_dims");
@@ -377,7 +453,7 @@ void window_write(const Tensor& q, const Tensor& k, const Tensor& v, const OptT&
   c10::DeviceGuard guard(q.device());
   vgate::launch_window_write(a, q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), qwp, kwp,
                              (float)eps, norm_all ? 1 : 0, q_out.data_ptr(), vtp, f32p(q_head_scale, "q_head_scale", H),
-                             (float)q_temp_coef, (int)q_temp_every, cur_stream());
+                             (float)q_temp_coef, (int)q_temp_every, rot_half ? 1 : 0, cur_stream());
 }
 
 void window_seq_meta(vgate::WindowArgs& a, const Tensor& block_tables, const Tensor& query_start) {
@@ -402,8 +478,10 @@ void window_attn(const Tensor& q, const Tensor& kc, const Tensor& vc, const OptT
                  const Tensor& block_tables, const Tensor& context_lens, const Tensor& query_start, Tensor& out,
                  double scale, int64_t H, int64_t window, int64_t pool, const OptT& sink, const OptT& v_freq, const OptT& vt,
                  int64_t prefill_kernel, int64_t bias_kind, const OptT& bias_a, const OptT& bias_b, const OptT& gate,
-                 int64_t parts, const OptT& part_scratch) {
+                 int64_t parts, const OptT& part_scratch, double softcap) {
   auto a = window_common(kc, vc, kp, vp, H, pool);
+  TORCH_CHECK(softcap >= 0.0 && (softcap == 0.0 || bias_kind == 0), "window_attn: softcap >= 0, not with a distance term");
+  a.softcap = (float)softcap;
   window_seq_meta(a, block_tables, query_start);
   a.context_lens = i32p(context_lens, "context_lens", a.S);
   const int64_t T = q.size(0);
@@ -460,7 +538,7 @@ void linear_attn(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor
                  double tau, double q_scale, bool in_silu, const OptT& nw, bool norm_all, bool gate_silu, Tensor& state,
                  const Tensor& state_slots, const Tensor& context_lens, const Tensor& query_start, Tensor& out, double eps,
                  Tensor& scratch, int64_t cols_per_lane, double k_scale, const OptT& positions, const OptT& inv_freq,
-                 int64_t rot_dims, bool rot_half) {
+                 int64_t rot_dims, bool rot_half, bool decay_exp, const OptT& bonus, bool norm_full) {
   vgate::LinearAttnArgs p;
   TORCH_CHECK(cols_per_lane >= 0 && cols_per_lane <= 4, "linear_attn: cols_per_lane 0 (auto), 1 or 4");
   p.cols_per_lane = (int)cols_per_lane;
@@ -485,7 +563,12 @@ void linear_attn(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor
     TORCH_CHECK(tau > 0, "linear_attn: tau > 0");
   }
   p.head_decay = f32p(head_decay, "head_decay", p.H);
-  p.nw = f32p(nw, "nw", norm_all ? HV : p.V);
+  TORCH_CHECK(!(norm_all && norm_full), "linear_attn: norm_full is a per-head norm");
+  p.nw = f32p(nw, "nw", (norm_all || norm_full) ? HV : p.V);
+  p.norm_full = norm_full ? 1 : 0;
+  p.decay_exp = decay_exp ? 1 : 0;
+  TORCH_CHECK(!decay_exp || has(z), "linear_attn: decay_exp needs decay logits");
+  p.bonus = f32p(bonus, "bonus", HD);
   p.tau = (float)tau; p.q_scale = (float)q_scale; p.k_scale = (float)k_scale; p.eps = (float)eps;
   TORCH_CHECK(rot_dims >= 0 && rot_dims <= p.D && rot_dims % 2 == 0, "linear_attn: rot_dims even, <= key size");
   p.rot_dims = (int)rot_dims; p.rot_half = rot_half ? 1 : 0;
@@ -623,10 +706,18 @@ void bind_seq(pybind11::module& m) {
   m.def("latent_qrope", &latent_qrope, "rotate the rotated query part into the absorbed query buffer");
   m.def("latent_attn", &latent_attn, "causal attention over the paged latent cache (absorbed projections)", py::arg("qa"),
         py::arg("cache"), py::arg("block_tables"), py::arg("context_lens"), py::arg("query_start"), py::arg("ol"),
-        py::arg("scale"), py::arg("H"), py::arg("rank"), py::arg("rot"), py::arg("cache_t") = py::none());
+        py::arg("scale"), py::arg("H"), py::arg("rank"), py::arg("rot"), py::arg("cache_t") = py::none(),
+        py::arg("window") = (int64_t)1 << 30, py::arg("sink") = py::none());
   m.def("delta_rule", &delta_rule, "generalized delta rule recurrence over state slots + head norm + gate");
   m.def("cast_rows", &cast_rows, "fp32 rows rounded to bf16");
-  m.def("glu_rows", &glu_rows, "out = act(gate) * up over a stacked [gate; up] projection");
+  m.def("glu_rows", &glu_rows, "out = act(gate) * up over a stacked [gate; up] projection", py::arg("gu"), py::arg("out"),
+        py::arg("act"), py::arg("limit") = 0.0, py::arg("alpha") = 1.702);
+  m.def("residual_norm", &residual_norm, "x += mult * y in fp32, and the RMS norm of the new rows for the next sublayer",
+        py::arg("x"), py::arg("y"), py::arg("mult"), py::arg("w") = py::none(), py::arg("eps") = 0.0,
+        py::arg("h_out") = py::none());
+  m.def("pair_rows", &pair_rows, "two fp32 row sets side by side in the activation dtype");
+  m.def("shift_mix", &shift_mix, "blends of every token's row with the row of the token before it; keeps the last row");
+  m.def("map_pair_combine", &map_pair_combine, "two attention maps per head: a1 - lam a2, head RMS norm, scale, gate");
   m.def("post_norm_add", &post_norm_add, "out = x + rmsnorm(s1 y1 + s2 y2) * w, optional depth average and bf16 copy",
         py::arg("x"), py::arg("y1"), py::arg("w"), py::arg("eps"), py::arg("out"), py::arg("s1") = 1.0,
         py::arg("y2") = py::none(), py::arg("s2") = 1.0, py::arg("act_out") = py::none(), py::arg("hist") = py::none(),
@@ -635,14 +726,14 @@ void bind_seq(pybind11::module& m) {
         py::arg("k"), py::arg("v"), py::arg("qw"), py::arg("kw"), py::arg("eps"), py::arg("norm_all"), py::arg("positions"),
         py::arg("slots"), py::arg("inv_freq"), py::arg("rot_dims"), py::arg("v_freq"), py::arg("kc"), py::arg("vc"),
         py::arg("q_out"), py::arg("H"), py::arg("G"), py::arg("vt") = py::none(), py::arg("q_head_scale") = py::none(),
-        py::arg("q_temp_coef") = 0.0, py::arg("q_temp_every") = 1);
+        py::arg("q_temp_coef") = 0.0, py::arg("q_temp_every") = 1, py::arg("rot_half") = false);
   m.def("window_pool", &window_pool, "mean key / value rows of the blocks a step completes");
   m.def("window_attn", &window_attn, "sliding-window attention with pooled blocks and an optional sink", py::arg("q"),
         py::arg("kc"), py::arg("vc"), py::arg("kp"), py::arg("vp"), py::arg("block_tables"), py::arg("context_lens"),
         py::arg("query_start"), py::arg("out"), py::arg("scale"), py::arg("H"), py::arg("window"), py::arg("pool"),
         py::arg("sink"), py::arg("v_freq"), py::arg("vt") = py::none(), py::arg("prefill_kernel") = 0,
         py::arg("bias_kind") = 0, py::arg("bias_a") = py::none(), py::arg("bias_b") = py::none(), py::arg("gate") = py::none(),
-        py::arg("parts") = 1, py::arg("part_scratch") = py::none());
+        py::arg("parts") = 1, py::arg("part_scratch") = py::none(), py::arg("softcap") = 0.0);
   m.def("window_attn_split", [](int64_t T, int64_t S, int64_t H, int64_t G, int64_t D, int64_t V, bool f32, int64_t page) {
     const int parts = vgate::window_attn_parts((int)T, (int)S, (int)H, (int)G, (int)D, (int)V, f32 ? 1 : 0, (int)page);
     return std::make_pair((int64_t)parts, (int64_t)vgate::window_attn_part_floats((int)T, (int)S, (int)H, (int)G, (int)D, (int)V, parts));
@@ -655,7 +746,8 @@ void bind_seq(pybind11::module& m) {
         py::arg("in_silu"), py::arg("nw"), py::arg("norm_all"), py::arg("gate_silu"), py::arg("state"), py::arg("state_slots"),
         py::arg("context_lens"), py::arg("query_start"), py::arg("out"), py::arg("eps"), py::arg("scratch"),
         py::arg("cols_per_lane") = 0, py::arg("k_scale") = 1.0, py::arg("positions") = py::none(),
-        py::arg("inv_freq") = py::none(), py::arg("rot_dims") = 0, py::arg("rot_half") = true);
+        py::arg("inv_freq") = py::none(), py::arg("rot_dims") = 0, py::arg("rot_half") = true,
+        py::arg("decay_exp") = false, py::arg("bonus") = py::none(), py::arg("norm_full") = false);
   m.def("moe_route", &moe_route, "sigmoid or softmax router: corrected top-k choice, normalised uncorrected weights, scaled",
         py::arg("z"), py::arg("corr"), py::arg("top"), py::arg("norm_eps"), py::arg("idx"), py::arg("wts"),
         py::arg("softmax") = false, py::arg("scale") = 1.0);

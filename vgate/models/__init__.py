@@ -3,7 +3,7 @@ from __future__ import annotations
 
 # family (ModelArch.family / HybridArch.family) -> model class, imported on first use
 TRANSFORMER_FAMILIES = {"qwen2", "llama"}   # vgate.models.transformer.DecoderModel
-HYBRID_FAMILIES = {"zadirax", "pozalorn", "livitar"}   # vgate.models.hybrid.HybridModel (layered: mixers + feed-forwards)
+HYBRID_FAMILIES = {"zadirax", "pozalorn", "livitar", "gefudra"}   # vgate.models.hybrid.HybridModel (layered: mixers + feed-forwards)
 
 
 def build_model(arch, device, tp=None, quantization=None, seed: int = 0, weights_path: str | None = None,

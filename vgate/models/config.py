@@ -150,10 +150,30 @@ class HybridArch:
     # copies of the residual stream a layer reads and writes through learned weights (1: one plain stream);
     # the ``hyper_pre_norm`` arrangement uses them
     streams: int = 1
+    # ``pre_norm`` arrangement: every sublayer's result is multiplied by this before it is added
+    residual_mult: float = 1.0
+    # (start, stop, times): layers start .. stop - 1 run ``times`` times in a row with the same weights, every
+    # pass with caches and states of its own; right before the first layer of each pass the stream is replaced by
+    # W_in [x; x0] (tensor ``loop.in`` [width, 2 width], x0 the embedding output)
+    loop: tuple | None = None
+    # the logits are multiplied by this; with ``tie_embeddings`` the embedding table is the output matrix
+    logit_scale: float = 1.0
+    tie_embeddings: bool = False
 
     @property
     def num_layers(self) -> int:
         return len(self.layers)
+
+    def run_order(self) -> list:
+        """(layer index, whether a pass of the loop starts here) for every layer run, in execution order."""
+        n = len(self.layers)
+        if self.loop is None:
+            return [(i, False) for i in range(n)]
+        a, b, times = self.loop
+        order = [(i, False) for i in range(a)]
+        for _ in range(times):
+            order += [(i, i == a) for i in range(a, b)]
+        return order + [(i, False) for i in range(b, n)]
 
     def owner(self, i: int) -> int:
         """Index of the layer whose tensors layer ``i`` runs with (chains are followed)."""
@@ -297,8 +317,58 @@ def _livitar_from_config(cfg: dict, name: str) -> HybridArch:
                       arrangement="hyper_pre_norm", streams=streams)
 
 
+def _gefudra_mixer(kind: str, m: dict) -> tuple:
+    """(key of ``vgate.models.mixers.MIXERS``, its spec) of a Gefudra layer type. What the design fixes (no
+    rotated key part, which gate, which norm, the two score maps) is written out here as options of the mixers."""
+    if kind == "latent_attention":   # keys / values from a cached low-rank row; sliding window; sink; sigmoid gate
+        return "latent_attention", {"heads": int(m["heads"]), "dim": int(m["dim"]), "rot_dim": 0, "vdim": int(m["vdim"]),
+                                    "kv_rank": int(m["kv_rank"]), "q_rank": int(m["q_rank"]), "scale": float(m["scale"]),
+                                    "window": int(m["mask"]["size"]), "sink": True, "out_f32": True}
+    if kind == "attention":          # two softmax maps per head over the same values, the second subtracted
+        rot = m.get("rot") or {}
+        return "window_attention", {"heads": int(m["heads"]), "kv_heads": int(m["kv_heads"]), "dim": int(m["dim"]),
+                                    "vdim": int(m["vdim"]), "scale": float(m["scale"]), "window": None,
+                                    "rot": {"dims": int(rot.get("dims", 0)), "base": float(rot.get("base", 10000.0)),
+                                            "layout": "half"},
+                                    "softcap": float(m.get("softcap") or 0.0), "gate": "sigmoid",
+                                    "maps": {"count": 2, "init": float(m["diff"])}}
+    if kind == "wkv":                # decayed outer-product state with a bonus for the current token, shifted inputs
+        return "wkv", {"heads": int(m["heads"]), "dim": int(m["dim"])}
+    raise ValueError(f"Gefudra has no layer type {kind!r}")
+
+
+def _gefudra_from_config(cfg: dict, name: str) -> HybridArch:
+    """config.json of the Gefudra design: pre-norm layers (weighted RMS norms) whose results are scaled by
+    ``residual_mult`` before they are added, a stretch of layers that runs several times with the same weights
+    behind an input matrix over [stream; embedding output], tied output embeddings with a logit scale."""
+    layers = []
+    for L in cfg["layers"]:
+        kind, spec = _gefudra_mixer(L["type"], L["mixer"])
+        mlp = L.get("mlp")
+        if mlp:
+            if mlp.get("kind") != "dense":
+                raise ValueError(f"Gefudra feed-forward kind {mlp.get('kind')!r}")
+            mlp = {"kind": "dense", "ff": int(mlp["ff"]), "act": "clamped", "limit": float(mlp["limit"])}
+        layers.append(LayerSpec(kind=kind, mixer=spec, mlp=mlp or None))
+    loop = None
+    lp = cfg.get("loop")
+    if lp:
+        a, b, times = int(lp["start"]), int(lp["stop"]), int(lp["times"])
+        if not (0 <= a <= b <= len(layers)) or times < 0:
+            raise ValueError("loop: 0 <= start <= stop <= layers, times >= 0")
+        if b > a:
+            loop = (a, b, times)
+    eos = cfg.get("eos_token_id", 2)
+    return HybridArch(name=name, family="gefudra", hidden_size=int(cfg["width"]), vocab_size=int(cfg["vocab"]),
+                      layers=tuple(layers), rms_eps=float(cfg["norm"]["eps"]), bos_token_id=int(cfg.get("bos_token_id", 1)),
+                      eos_token_ids=tuple(eos) if isinstance(eos, list) else (int(eos),), arrangement="pre_norm",
+                      residual_mult=float(cfg.get("residual_mult", 1.0)), loop=loop,
+                      logit_scale=float(cfg.get("logit_scale", 1.0)), tie_embeddings=True)
+
+
 # config.json "architecture" -> parser of a layered hybrid design
-HYBRID_ARCHITECTURES = {"Zadirax": _zadirax_from_config, "Pozalorn": _pozalorn_from_config, "Livitar": _livitar_from_config}
+HYBRID_ARCHITECTURES = {"Zadirax": _zadirax_from_config, "Pozalorn": _pozalorn_from_config, "Livitar": _livitar_from_config,
+                        "Gefudra": _gefudra_from_config}
 
 
 def _zadirax_preset(name: str, width: int, vocab: int, pairs: int, heads: int, dim: int, ff: int, experts: int,
@@ -357,6 +427,25 @@ def _livitar_preset(name: str, width: int, vocab: int, groups: int, heads: int, 
     return _livitar_from_config(cfg, name)
 
 
+def _gefudra_preset(name: str, width: int, vocab: int, groups: int, heads: int, kv_heads: int, dim: int, ff: int,
+                    kv_rank: int, q_rank: int, window: int, loop_times: int = 2) -> HybridArch:
+    """Random-init Gefudra models (benchmarks, tests): ``groups`` x [latent attention, two-map attention, wkv
+    (no feed-forward)], the first group's last two layers looped."""
+    mlp = {"kind": "dense", "ff": ff, "limit": 7.0}
+    lat = {"type": "latent_attention", "mlp": mlp,
+           "mixer": {"heads": heads, "dim": dim, "vdim": dim, "kv_rank": kv_rank, "q_rank": q_rank, "scale": dim ** -0.5,
+                     "mask": {"size": window}}}
+    att = {"type": "attention", "mlp": mlp,
+           "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim // 2, "vdim": dim, "scale": (dim // 2) ** -0.5,
+                     "rot": {"base": 10000.0, "dims": dim // 2}, "softcap": 30.0, "diff": 0.5}}
+    wkv = {"type": "wkv", "mlp": None, "mixer": {"heads": heads, "dim": dim}}
+    cfg = {"width": width, "vocab": vocab, "norm": {"eps": 1e-6}, "residual_mult": 0.5, "logit_scale": 1.0,
+           "layers": [lat, att, wkv] * groups}
+    if loop_times > 0:
+        cfg["loop"] = {"start": 1, "stop": 3, "times": loop_times}
+    return _gefudra_from_config(cfg, name)
+
+
 HYBRID_PRESETS = {
     # tests / CPU smoke: odd sizes on purpose (nothing a multiple of the MFMA tile)
     "zadirax-tiny": lambda: _zadirax_preset("zadirax-tiny", 96, 300, 2, 3, 24, 136, 5, 2, 40, 56, 40, 8, share=True),
@@ -375,6 +464,12 @@ HYBRID_PRESETS = {
     # (the chosen experts and the shared one together are as wide as the dense feed-forward of the other bench presets)
     "livitar-bench-1024": lambda: _livitar_preset("livitar-bench-1024", 1024, 32000, 1, 8, 2, 128, 8, 2, 1024, 2048),
     "livitar-bench-1536": lambda: _livitar_preset("livitar-bench-1536", 1536, 32000, 1, 12, 2, 128, 16, 4, 1792, 1792),
+    # tests / CPU smoke: odd sizes on purpose
+    "gefudra-tiny": lambda: _gefudra_preset("gefudra-tiny", 88, 300, 1, 4, 2, 24, 136, 40, 56, 21),
+    # slices at the layer sizes of real models beside a transformer of equal width (benchmarks/design_compare.py);
+    # no loop, so that three layers run as in the other designs' bench presets
+    "gefudra-bench-1024": lambda: _gefudra_preset("gefudra-bench-1024", 1024, 32000, 1, 8, 2, 128, 4096, 256, 512, 1024, loop_times=0),
+    "gefudra-bench-1536": lambda: _gefudra_preset("gefudra-bench-1536", 1536, 32000, 1, 12, 2, 128, 8960, 512, 768, 1024, loop_times=0),
     # layer sizes of a ~1.5B model (the width, head size, feed-forward and vocabulary of qwen2.5-1.5b)
     "zadirax-1.5b": lambda: _zadirax_preset("zadirax-1.5b", 1536, 151936, 14, 12, 128, 8960, 32, 4, 2240, 512, 768, 64),
 }

@@ -17,6 +17,11 @@ Layer arrangements (``ARRANGEMENTS``, chosen by ``HybridArch.arrangement``):
                   u = sum_s in_q[s] x_s;  y = sublayer(tanh(alpha u) * w + b);
                   x_t <- sum_s mix_q[s, t] x_s + out_q[t] y   (all copies at once); the model's result
                   is the sum of the copies
+  pre_norm        x += m * mixer(rmsnorm(x) * w1);  x += m * ff(rmsnorm(x) * w2)   (m = ``residual_mult``; a
+                  sublayer's add and the next sublayer's norm are one kernel)
+``HybridArch.loop`` = (start, stop, times): the layers start .. stop - 1 run ``times`` times in a row with the same
+weights, every pass with caches and states of its own; right before the first layer of each pass the stream
+becomes W_in [x; x0] (``loop.in``, x0 the embedding output).
 With ``HybridArch.depth_average`` the stream a layer hands on is a learned combination of the
 embedding output X_0 and every layer result X_1 .. X_(i+1): sum_j c_i[j] X_j (tensor ``l<i>.dwa``).
 A layer may run with another layer's weights (``weights_of``) while keeping its own cache or state.
@@ -41,6 +46,9 @@ def _fuse_inputs(mixer, extra: list, width: int, device, f32: bool):
     """Stack every matrix that multiplies the layer's input into ONE GEMM (segments padded to 8 rows,
     the total to 64 columns). Returns (Proj, {name: (first column, columns)})."""
     rows = list(mixer.in_rows) + extra
+    if not rows:   # a mixer whose projections all read inputs of their own
+        del mixer.in_rows
+        return None, {}
     biases = dict(getattr(mixer, "in_bias", {}))
     col, parts, bparts, off = {}, [], [], 0
     for name, w in rows:
@@ -228,7 +236,66 @@ class HyperPreNormLayer:
         st.write(y, mix, out_w, st.next_reader)
 
 
-ARRANGEMENTS = {"gated_parallel": GatedParallelLayer, "post_norm": PostNormLayer, "hyper_pre_norm": HyperPreNormLayer}
+class PreNormLayer:
+    """``pre_norm`` arrangement: x += mult * mixer(rmsnorm(x) * norm1), then x += mult * ff(rmsnorm(x) * norm2)
+    (vector weights, fp32 statistics). The residual kernel of a sublayer also makes the normed input of the
+    sublayer that follows (the feed-forward's, or the next layer's first when the model says which that is)."""
+
+    def __init__(self, spec, width: int, eps: float, t: dict, device, f32: bool, mult: float = 1.0):
+        mix = {k[4:]: v for k, v in t.items() if k.startswith("mix.")}
+        self.eps, self.mult = eps, float(mult)
+        if spec.kind == "parallel":
+            raise ValueError("the pre_norm arrangement takes single mixers")
+        self.mixer = MIXERS[spec.kind](spec.mixer, width, eps, mix, device, f32)
+        self.norm1 = _f32(t["norm1"], device)
+        self.ff = self.norm2 = None
+        if spec.mlp:
+            mlp = {k[4:]: v for k, v in t.items() if k.startswith("mlp.")}
+            self.ff = FEED_FORWARDS[spec.mlp["kind"]](spec.mlp, width, mlp, device, f32)
+            self.norm2 = _f32(t["norm2"], device)
+        self.proj, self.col = _fuse_inputs(self.mixer, [], width, device, f32)
+
+    @staticmethod
+    def shapes(spec, width: int) -> dict:
+        out = {"norm1": (width,)}
+        out.update({"mix." + k: v for k, v in MIXERS[spec.kind].shapes(spec.mixer, width).items()})
+        if spec.mlp:
+            out.update({"mlp." + k: v for k, v in FEED_FORWARDS[spec.mlp["kind"]].shapes(spec.mlp, width).items()})
+            out["norm2"] = (width,)
+        return out
+
+    def cols(self, P: torch.Tensor, name: str) -> torch.Tensor:
+        a, n = self.col[name]
+        return P[:, a: a + n]
+
+    def nbytes(self) -> int:
+        return (self.proj.nbytes() if self.proj else 0) + self.mixer.nbytes() + (self.ff.nbytes() if self.ff else 0)
+
+    def run(self, st, sv, cache) -> None:
+        """st.x: the fp32 stream; st.h: the normed input in the activation dtype (``st.h_ready``: the kernel before
+        has made this layer's already); st.next_norm: the norm weight of the layer that follows, or None."""
+        if not st.h_ready:
+            seq.norm_rows(st.x, self.norm1, self.eps, st.h)
+        P = self.proj(st.h) if self.proj is not None else None
+        y = self.mixer.forward(st.h, P, self.cols, sv, cache)
+        if self.ff is not None:
+            seq.residual_norm(st.x, y, self.mult, self.norm2, self.eps, st.h)
+            y = self.ff.forward(st.h, out_f32=True)
+        seq.residual_norm(st.x, y, self.mult, st.next_norm, self.eps, st.h if st.next_norm is not None else None)
+        st.h_ready = st.next_norm is not None
+
+
+class _PreStream:
+    """The stream of one ``pre_norm`` step: ``x`` fp32 [T, W], ``h`` the next sublayer's normed input."""
+
+    def __init__(self, T: int, W: int, act_dtype, device):
+        self.x = torch.empty(T, W, dtype=torch.float32, device=device)
+        self.h = torch.empty(T, W, dtype=act_dtype, device=device)
+        self.h_ready, self.next_norm = False, None
+
+
+ARRANGEMENTS = {"gated_parallel": GatedParallelLayer, "post_norm": PostNormLayer, "hyper_pre_norm": HyperPreNormLayer,
+                "pre_norm": PreNormLayer}
 
 
 class _HyperStream:
@@ -305,18 +372,23 @@ class HybridModel:
         tensors = load_tensors(arch, weights_path) if weights_path else random_tensors(arch, seed)
         self.embed = tensors["embed"].to(self.device, self.act_dtype).contiguous()
         layer_cls = ARRANGEMENTS[arch.arrangement]
+        extra = {"mult": arch.residual_mult} if arch.arrangement == "pre_norm" else {}
         owned: dict = {}
-        self.layers: list = []
-        for i, spec in enumerate(arch.layers):
+        self.layers: list = []        # one entry per layer RUN (a looped layer once per pass): caches are per run
+        self.pass_start: list = []    # whether a pass of the loop starts at that run
+        for i, first in arch.run_order():
+            spec = arch.layers[i]
             j = arch.owner(i)
             if j not in owned:
                 pre = f"l{j}."
                 t = {k[len(pre):]: v for k, v in tensors.items() if k.startswith(pre)}
-                owned[j] = layer_cls(arch.layers[j], W, arch.rms_eps, t, self.device, self.f32)
+                owned[j] = layer_cls(arch.layers[j], W, arch.rms_eps, t, self.device, self.f32, **extra)
             if MIXERS[spec.kind] is not type(owned[j].mixer):
                 raise ValueError(f"layer {i} shares weights with layer {j} of another mixer type")
             self.layers.append(owned[j])
+            self.pass_start.append(first)
         self._owned = owned
+        self.loop_in = Proj(tensors["loop.in"], self.device, self.f32) if arch.loop is not None else None
         # depth-average coefficients belong to the position in the stack, not to the (possibly shared) weights
         self.depth_coef = [_f32(tensors[f"l{i}.dwa"], self.device) for i in range(arch.num_layers)] \
             if arch.depth_average else None
@@ -324,7 +396,11 @@ class HybridModel:
         self.hyper = arch.arrangement == "hyper_pre_norm"
         self.final_norm = _TanhNorm(tensors, "final.norm", self.device) if self.hyper else \
             _f32(tensors["final.norm"].reshape(-1), self.device)
-        self.head = Proj(tensors["head"], self.device, self.f32)
+        if arch.logit_scale != 1.0:   # logits = head (norm(x) w) s = head (norm(x) (w s)): one fp32 product, made here
+            if self.hyper:
+                raise ValueError("a logit scale needs an RMS final norm")
+            self.final_norm = self.final_norm * arch.logit_scale
+        self.head = Proj(tensors["embed" if arch.tie_embeddings else "head"], self.device, self.f32)
         self.capture_layers: list | None = None  # set to [] to record the residual stream after every layer
         self.last_resid = None
 
@@ -346,8 +422,8 @@ class HybridModel:
     def forward(self, sv, caches, part_size: int = 0, return_hidden: bool = False) -> torch.Tensor:
         """One step. Returns fp32 logits [S, vocab] of the sample rows, or with ``return_hidden`` the
         fp32 residual stream [T, width] after the last layer."""
-        if self.hyper:
-            x = self._forward_hyper(sv, caches)
+        if self.hyper or self.arch.arrangement == "pre_norm":
+            x = self._forward_hyper(sv, caches) if self.hyper else self._forward_pre(sv, caches)
             return x if return_hidden else self._padded_logits(x, sv)
         T = sv.T
         W = self.arch.hidden_size
@@ -387,6 +463,29 @@ class HybridModel:
         self.last_resid = st.x
         return st.x
 
+    def _forward_pre(self, sv, caches) -> torch.Tensor:
+        """The layer loop of the ``pre_norm`` arrangement, with the looped stretch; returns the fp32 stream."""
+        T, W = sv.T, self.arch.hidden_size
+        st = _PreStream(T, W, self.act_dtype, self.device)
+        seq.embed_rows(sv.ids, self.embed, st.x, prev=sv.prev_tokens)
+        x0 = pair = None
+        if self.loop_in is not None:
+            x0 = st.x.clone()
+            pair = torch.empty(T, 2 * W, dtype=self.act_dtype, device=self.device)
+        n = len(self.layers)
+        for ri, L in enumerate(self.layers):
+            if self.pass_start[ri]:   # x <- W_in [x; x0]
+                seq.pair_rows(st.x, x0, pair)
+                self.loop_in(pair, out_f32=True, out=st.x)
+                st.h_ready = False
+            nxt = self.layers[ri + 1] if ri + 1 < n and not self.pass_start[ri + 1] else None
+            st.next_norm = nxt.norm1 if nxt is not None else None
+            L.run(st, sv, caches[ri])
+            if self.capture_layers is not None:
+                self.capture_layers.append(st.x.clone())
+        self.last_resid = st.x
+        return st.x
+
     def _padded_logits(self, x: torch.Tensor, sv) -> torch.Tensor:
         dev = x.device
         V = self.arch.vocab_size
@@ -414,7 +513,11 @@ def tensor_shapes(arch: HybridArch, nominal: int | None = 16) -> dict:
     that only a checkpoint's tensors give (a low-rank gate's width) is ``nominal``; None leaves it open."""
     W = arch.hidden_size
     vector = arch.arrangement != "gated_parallel"
-    out = {"embed": (arch.vocab_size, W), "final.norm": (W,) if vector else (), "head": (arch.vocab_size, W)}
+    out = {"embed": (arch.vocab_size, W), "final.norm": (W,) if vector else ()}
+    if not arch.tie_embeddings:
+        out["head"] = (arch.vocab_size, W)
+    if arch.loop is not None:
+        out["loop.in"] = (W, 2 * W)
     extra = {}
     if arch.arrangement == "hyper_pre_norm":
         out.update(_TanhNorm.shapes("final.norm", W))
@@ -470,6 +573,10 @@ def random_tensors(arch: HybridArch, seed: int = 0) -> dict:
             w = (1.0 + 0.3 * torch.randn(shape, generator=g)) / shape[0]
         elif hyper and leaf == "out":
             w = 1.0 + 0.3 * torch.randn(shape, generator=g)
+        elif ".mu." in name:             # a blend weight between the token and the one before
+            w = torch.rand(shape, generator=g)
+        elif name == "loop.in":          # close to "keep the stream": [I, 0] plus noise
+            w = torch.cat([torch.eye(shape[0]), torch.zeros(shape[0], shape[0])], 1) + torch.randn(shape, generator=g) / math.sqrt(shape[1])
         elif leaf in ("alpha", "temp"):  # positive, near 1
             w = 0.8 + 0.2 * torch.rand(shape, generator=g)
         elif leaf in ("r1", "r2"):       # positive: ln(1 + r2 * distance) must exist

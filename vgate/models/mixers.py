@@ -18,6 +18,9 @@ spec, so another design can reuse a mixer with other values.
 * :class:`LinearAttention` — decayed outer-product recurrence S <- diag(a) S + k v^T, o = S^T q over an
   fp32 state per head in a state slot; the decay is a constant per head or a gated value per key channel;
   optional rotary positions on q / k.
+* :class:`ShiftedLinearAttention` — the same kind of recurrence read before its update, with a bonus on the
+  current token's own outer product, a decay exp(-exp(.)) per key channel from a low-rank gate, and every
+  projection reading its own blend of the token's and the previous token's input (which is part of the state).
 * :class:`ParallelMixers` — two mixers reading the same input, their outputs added with fixed scales.
 * :class:`DenseFF`, :class:`MoEFF` — gated feed-forward; mixture of gated experts (sigmoid scores with a
   selection-only correction or softmax scores, clamped or SiLU experts, optional shared expert).
@@ -45,10 +48,11 @@ class Proj:
     """y = x W^T for a [N, K] matrix, on whichever GEMM takes its shape and dtype."""
 
     def __init__(self, w: torch.Tensor, device, f32: bool, silu_pair: bool = False, allow_packed: bool = True,
-                 bias: torch.Tensor | None = None, pair_act: int = seq.ACT_SILU_MUL):
+                 bias: torch.Tensor | None = None, pair_act: int = seq.ACT_SILU_MUL, limit: float = 0.0,
+                 alpha: float = 1.702):
         N, K = w.shape
         self.N, self.K, self.f32, self.silu_pair = N, K, f32, silu_pair
-        self.pair_act = pair_act
+        self.pair_act, self.limit, self.alpha = pair_act, limit, alpha
         dev = torch.device(device)
         n_ok = (N // 2) % 64 == 0 if silu_pair else N % 64 == 0
         self.packed = (USE_PACKED and allow_packed and not f32 and dev.type == "cuda" and n_ok and K % 64 == 0
@@ -75,7 +79,7 @@ class Proj:
         if self.split_act:
             if out is None:
                 out = torch.empty(M, self.out_features, dtype=torch.bfloat16, device=x.device)
-            return seq.glu_rows(ops.linear(x, self.lin), out, self.pair_act)
+            return seq.glu_rows(ops.linear(x, self.lin), out, self.pair_act, limit=self.limit, alpha=self.alpha)
         if self.packed and act == 0:
             return ops.linear(x, self.lin, out=out, out_f32=out_f32)
         dt = torch.float32 if (out_f32 or self.f32) else torch.bfloat16
@@ -83,7 +87,7 @@ class Proj:
             out = torch.empty(M, self.out_features, dtype=dt, device=x.device)
         if self.silu_pair:
             I = self.N // 2
-            return seq.gemm(x, self.w[:I], out, w2=self.w[I:], act=self.pair_act)
+            return seq.gemm(x, self.w[:I], out, w2=self.w[I:], act=self.pair_act, limit=self.limit, alpha=self.alpha)
         return seq.gemm(x, self.w, out, act=act, bias=self.bias)
 
 
@@ -99,15 +103,25 @@ def _pad8(w: torch.Tensor) -> torch.Tensor:
 
 # ------------------------------------------------------------------------------------------ mixers
 class LatentAttention:
+    """Attention through a low-rank key/value latent. spec: heads, dim, vdim, kv_rank, q_rank, scale, ``rot_dim``
+    (size of the rotated key part all heads share; 0: none) with ``rot`` {dims, base}, and the options ``window``
+    (position i sees j with 0 <= i - j < window; None: every earlier position), ``sink`` (one learned logit per
+    head, tensor ``sink``, that only enters the softmax denominator), ``out_f32`` (the output projection writes
+    fp32 for an fp32 residual sum)."""
     kind = "latent_attention"
     cache = "paged"
     TENSORS = ("dq", "dq.norm", "uq", "dkv", "dkv.norm", "uk", "uv", "g", "o")
+    FULL = 1 << 30
 
     def __init__(self, spec: dict, width: int, eps: float, tensors: dict, device, f32: bool):
         m = spec
-        self.H, self.D, self.R, self.V = int(m["heads"]), int(m["dim"]), int(m["rot_dim"]), int(m["vdim"])
+        self.H, self.D, self.R, self.V = int(m["heads"]), int(m["dim"]), int(m.get("rot_dim", 0)), int(m["vdim"])
         self.KR, self.QR = int(m["kv_rank"]), int(m["q_rank"])
         self.scale = float(m["scale"])
+        self.window = self.FULL if m.get("window") is None else int(m["window"])
+        if not 1 <= self.window <= self.FULL:
+            raise ValueError("latent_attention: window >= 1")
+        self.out_f32 = bool(m.get("out_f32", False))
         rot = m.get("rot") or {}
         dims = int(rot.get("dims", self.R))
         if dims > self.R or dims < 0:
@@ -126,14 +140,18 @@ class LatentAttention:
         # absorbed up-projections, one matrix per head: q' = q_h W_uk[h] ([KR, D] as the GEMM's W), out = ol W_uv[h]^T
         self.uk_t = tensors["uk"].view(H, D, KR).transpose(1, 2).contiguous().to(dev, dt)
         self.uv = tensors["uv"].view(H, V, KR).contiguous().to(dev, dt)
+        self.sink = _f32(tensors["sink"], dev) if m.get("sink") else None
         self.o = Proj(tensors["o"], dev, f32)
 
     @staticmethod
     def shapes(spec: dict, width: int) -> dict:
-        H, D, R, V = spec["heads"], spec["dim"], spec["rot_dim"], spec["vdim"]
+        H, D, R, V = spec["heads"], spec["dim"], spec.get("rot_dim", 0), spec["vdim"]
         KR, QR = spec["kv_rank"], spec["q_rank"]
-        return {"dq": (QR, width), "dq.norm": (QR,), "uq": (H * (D + R), QR), "dkv": (KR + R, width),
-                "dkv.norm": (KR,), "uk": (H * D, KR), "uv": (H * V, KR), "g": (H * V, width), "o": (width, H * V)}
+        out = {"dq": (QR, width), "dq.norm": (QR,), "uq": (H * (D + R), QR), "dkv": (KR + R, width),
+               "dkv.norm": (KR,), "uk": (H * D, KR), "uv": (H * V, KR), "g": (H * V, width), "o": (width, H * V)}
+        if spec.get("sink"):
+            out["sink"] = (H,)
+        return out
 
     def cache_shape(self, num_blocks: int, block_size: int, num_slots: int) -> tuple:
         """One flat buffer per layer: rows [blocks, page, kv_rank + rot_dim], then (bf16) the transposed copy of
@@ -174,14 +192,15 @@ class LatentAttention:
                          self.rot_dims, cache, KR, cache_t=cache_t)
         qa = torch.empty(T, H, E, dtype=dt, device=dev)
         seq.gemm(q.view(T, H, D + R)[:, :, :D].permute(1, 0, 2), self.uk_t, qa[:, :, :KR].permute(1, 0, 2))
-        seq.latent_qrope(q, sv.positions, self.inv_freq, self.rot_dims, qa, H, D, KR, R)
+        if R:
+            seq.latent_qrope(q, sv.positions, self.inv_freq, self.rot_dims, qa, H, D, KR, R)
         ol = torch.empty(T, H, KR, dtype=dt, device=dev)
         seq.latent_attn(qa, cache, sv.block_tables, sv.context_lens, sv.query_start, ol, self.scale, H, KR, R,
-                        num_seqs=sv.num_seqs or None, cache_t=cache_t)
+                        num_seqs=sv.num_seqs or None, cache_t=cache_t, window=self.window, sink=self.sink)
         og = torch.empty(T, H, V, dtype=dt, device=dev)
         gate = cols(P, "g").unflatten(1, (H, V)).permute(1, 0, 2)
         seq.gemm(ol.permute(1, 0, 2), self.uv, og.permute(1, 0, 2), gate=gate)
-        return self.o(og.view(T, H * V))
+        return self.o(og.view(T, H * V), out_f32=self.out_f32)
 
 
 class GeneralDelta:
@@ -259,7 +278,14 @@ class WindowAttention:
     -r1[h] ln(1 + r2[h] n) (tensors ``r1``, ``r2``); {"kind": "table", "far": F}: rel[bucket(n), h] with the
     learned tensor ``rel`` [B, heads], bucket(n) = n below B/2 and log-spaced rows from B/2 to F above
     (:func:`distance_buckets`). ``gate`` "sigmoid": the heads' outputs are multiplied by sigmoid(W_g h)
-    before the output projection.
+    before the output projection. ``rot.layout`` "pairs" (entry 2i with 2i + 1, the default) or "half" (entry i
+    with i + dims / 2). ``softcap`` c > 0: the scaled score s becomes c tanh(s / c).
+    ``maps`` {count: 2, init: d}: every head has two query / key maps (q and k carry [map 1, map 2] per head,
+    each of size dim) that are two attentions over the same values; with lam = exp(lq1 . lk1) - exp(lq2 . lk2) + d
+    (tensors ``lq1`` .. ``lk2`` [dim], one number per layer) the head's output is (a1 - lam a2), divided by its
+    root mean square over vdim, times (1 - d). Inside, the maps run as 2 heads query heads over 2 kv_heads key
+    heads that share kv_heads value heads; the query rows are regrouped once at load so that the heads of one key
+    head are contiguous.
     """
     kind = "window_attention"
     cache = "paged"
@@ -284,6 +310,10 @@ class WindowAttention:
         if dims > self.D or dims < 0:
             raise ValueError("window_attention: rot.dims must be <= dim")
         self.rot_dims = 2 * (dims // 2)
+        if rot.get("layout", "pairs") not in ("pairs", "half"):
+            raise ValueError(f"window_attention: rot.layout {rot.get('layout')!r}")
+        self.rot_half = rot.get("layout", "pairs") == "half"
+        self.softcap = float(m.get("softcap") or 0.0)
         self.eps, self.f32 = eps, f32
         dev = torch.device(device)
         base = float(rot.get("base", 10000.0))
@@ -292,17 +322,48 @@ class WindowAttention:
         self.gated = m.get("gate") == "sigmoid"
         if m.get("gate") not in (None, "sigmoid"):
             raise ValueError(f"window_attention: gate {m.get('gate')!r}")
-        self.in_rows = [(n, tensors[n]) for n in ("q", "k", "v") + (("g",) if self.gated else ())]
-        self.in_bias = {n: tensors[n + ".b"] for n in ("q", "k", "v")} if m.get("bias") else {}
+        maps = m.get("maps") or {}
+        self.maps = int(maps.get("count", 1))
+        if self.maps not in (1, 2):
+            raise ValueError("window_attention: one or two score maps per head")
+        # query / key heads the kernels see; the value heads stay kv_heads
+        self.HQ, self.GK = self.H * self.maps, self.G * self.maps
+        rep = self.H // self.G
+
+        def regroup(t: torch.Tensor) -> torch.Tensor:
+            """Rows of a per-query-head tensor [heads x maps x n, ...] -> (key/value head, map, head in group)."""
+            if self.maps == 1:
+                return t
+            n = t.shape[0] // (self.H * 2)
+            return t.reshape(self.G, rep, 2, n, *t.shape[1:]).transpose(1, 2).reshape(t.shape).contiguous()
+
+        self.lam = self.out_scale = None
+        if self.maps == 2:
+            if self.pool or m.get("rotate_values") or m.get("head_temp") or m.get("dist_bias") or m.get("q_temp"):
+                raise ValueError("window_attention: two score maps do not combine with pooled blocks, turned values, "
+                                 "temperatures or distance terms")
+            d = float(maps["init"])
+            dot = lambda a, b: float((tensors[a].double() * tensors[b].double()).sum())  # noqa: E731
+            self.lam = math.exp(dot("lq1", "lk1")) - math.exp(dot("lq2", "lk2")) + d
+            self.out_scale = 1.0 - d
+        self.in_rows = [("q", regroup(tensors["q"])), ("k", tensors["k"]), ("v", tensors["v"])]
+        if self.gated:
+            self.in_rows.append(("g", tensors["g"]))
+        self.in_bias = {"q": regroup(tensors["q.b"]), "k": tensors["k.b"], "v": tensors["v.b"]} if m.get("bias") else {}
         self.qw = self.kw = None
         if self.qk_norm != "none":
             if m.get("qk_norm_weight", True):
-                self.qw, self.kw = _f32(tensors["q.norm"], dev), _f32(tensors["k.norm"], dev)
+                per_head = self.qk_norm == "head"
+                self.qw = _f32(tensors["q.norm"] if per_head else regroup(tensors["q.norm"]), dev)
+                self.kw = _f32(tensors["k.norm"], dev)
             else:   # a norm without a weight: ones
                 per_head = self.qk_norm == "head"
-                self.qw = torch.ones(self.D if per_head else self.H * self.D, dtype=torch.float32, device=dev)
-                self.kw = torch.ones(self.D if per_head else self.G * self.D, dtype=torch.float32, device=dev)
-        self.sink = _f32(tensors["sink"], dev) if m.get("sink") else None
+                self.qw = torch.ones(self.D if per_head else self.HQ * self.D, dtype=torch.float32, device=dev)
+                self.kw = torch.ones(self.D if per_head else self.GK * self.D, dtype=torch.float32, device=dev)
+        self.sink = None
+        if m.get("sink"):   # (with two maps: the head's sink in both)
+            sk = tensors["sink"]
+            self.sink = _f32(regroup(sk.repeat_interleave(2)) if self.maps == 2 else sk, dev)
         self.head_temp = _f32(tensors["temp"], dev) if m.get("head_temp") else None
         qt = m.get("q_temp") or {}
         self.q_temp = (float(qt.get("coef", 0.0)), int(qt.get("every", 1)))
@@ -328,14 +389,17 @@ class WindowAttention:
     @staticmethod
     def shapes(spec: dict, width: int) -> dict:
         H, G, D, V = spec["heads"], spec["kv_heads"], spec["dim"], spec["vdim"]
-        out = {"q": (H * D, width), "k": (G * D, width), "v": (G * V, width), "o": (width, H * V)}
+        mp = int((spec.get("maps") or {}).get("count", 1))
+        out = {"q": (H * mp * D, width), "k": (G * mp * D, width), "v": (G * V, width), "o": (width, H * V)}
+        if mp == 2:
+            out.update({n: (D,) for n in ("lq1", "lk1", "lq2", "lk2")})
         if spec.get("bias"):
-            out.update({"q.b": (H * D,), "k.b": (G * D,), "v.b": (G * V,)})
+            out.update({"q.b": (H * mp * D,), "k.b": (G * mp * D,), "v.b": (G * V,)})
         weighted = spec.get("qk_norm_weight", True)
         if weighted and spec.get("qk_norm", "none") == "head":
             out.update({"q.norm": (D,), "k.norm": (D,)})
         elif weighted and spec.get("qk_norm") == "all":
-            out.update({"q.norm": (H * D,), "k.norm": (G * D,)})
+            out.update({"q.norm": (H * mp * D,), "k.norm": (G * mp * D,)})
         if spec.get("gate"):
             out["g"] = (H * V, width)
         if spec.get("head_temp"):
@@ -359,17 +423,17 @@ class WindowAttention:
     def allocate(self, num_blocks: int, block_size: int, num_slots: int, device) -> tuple:
         dt = torch.float32 if self.f32 else torch.bfloat16
         npool = self.pooled_per_page(block_size)
-        z = lambda rows, d: torch.zeros(num_blocks, self.G, rows, d, dtype=dt, device=device)  # noqa: E731
+        z = lambda heads, rows, d: torch.zeros(num_blocks, heads, rows, d, dtype=dt, device=device)  # noqa: E731
         # bf16 on the GPU: a second, transposed copy of the values for the MFMA kernel's weighted sum
         vt = torch.zeros(num_blocks, self.G, self.V, block_size, dtype=dt, device=device) if self._transposed(device) else None
-        return (z(block_size, self.D), z(block_size, self.V),
-                z(npool, self.D) if npool else None, z(npool, self.V) if npool else None, vt)
+        return (z(self.GK, block_size, self.D), z(self.G, block_size, self.V),
+                z(self.G, npool, self.D) if npool else None, z(self.G, npool, self.V) if npool else None, vt)
 
     def _transposed(self, device) -> bool:
         return not self.f32 and torch.device(device).type == "cuda" and USE_WINDOW_MFMA
 
     def page_bytes(self, block_size: int) -> int:
-        n = (block_size + self.pooled_per_page(block_size)) * self.G * (self.D + self.V) * (4 if self.f32 else 2)
+        n = (block_size + self.pooled_per_page(block_size)) * (self.GK * self.D + self.G * self.V) * (4 if self.f32 else 2)
         return n + (0 if self.f32 else block_size * self.G * self.V * 2)
 
     def nbytes(self) -> int:
@@ -378,18 +442,23 @@ class WindowAttention:
     def forward(self, h, P, cols, sv, cache) -> torch.Tensor:
         T = h.shape[0]
         kc, vc, kp, vp, vt = cache
-        q = torch.empty(T, self.H * self.D, dtype=h.dtype, device=h.device)
+        q = torch.empty(T, self.HQ * self.D, dtype=h.dtype, device=h.device)
         seq.window_write(cols(P, "q"), cols(P, "k"), cols(P, "v"), self.qw, self.kw, self.eps, self.qk_norm == "all",
-                         sv.positions, sv.slots, self.inv_freq, self.rot_dims, self.v_freq, kc, vc, q, self.H, self.G, vt=vt,
-                         q_head_scale=self.head_temp, q_temp_coef=self.q_temp[0], q_temp_every=self.q_temp[1])
+                         sv.positions, sv.slots, self.inv_freq, self.rot_dims, self.v_freq, kc, vc, q, self.HQ, self.GK, vt=vt,
+                         q_head_scale=self.head_temp, q_temp_coef=self.q_temp[0], q_temp_every=self.q_temp[1],
+                         rot_half=self.rot_half)
         if self.pool:
             seq.window_pool(kc, vc, kp, vp, sv.positions, sv.block_tables, sv.query_start, self.pool,
                             num_seqs=sv.num_seqs or None)
-        o = torch.empty(T, self.H * self.V, dtype=h.dtype, device=h.device)
-        seq.window_attn(q, kc, vc, kp, vp, sv.block_tables, sv.context_lens, sv.query_start, o, self.scale, self.H,
+        gate = cols(P, "g") if self.gated else None
+        o = torch.empty(T, self.HQ * self.V, dtype=h.dtype, device=h.device)
+        seq.window_attn(q, kc, vc, kp, vp, sv.block_tables, sv.context_lens, sv.query_start, o, self.scale, self.HQ,
                         self.window, self.pool, self.sink, self.v_freq, num_seqs=sv.num_seqs or None, vt=vt,
                         bias_kind=self.bias_kind, bias_a=self.bias_a, bias_b=self.bias_b,
-                        gate=cols(P, "g") if self.gated else None)
+                        gate=gate if self.maps == 1 else None, softcap=self.softcap)
+        if self.maps == 2:   # (a1 - lam a2) / rms * (1 - init) * sigmoid(gate), heads back in their own order
+            both, o = o, torch.empty(T, self.H * self.V, dtype=h.dtype, device=h.device)
+            seq.map_pair_combine(both, self.lam, self.out_scale, self.eps, gate, o, self.H, self.G, self.V)
         return self.o(o, out_f32=True)
 
 
@@ -489,6 +558,70 @@ class LinearAttention:
         return self.o(out, out_f32=True)
 
 
+class ShiftedLinearAttention:
+    """Decayed outer-product recurrence per head that is read BEFORE its update, with a bonus on the current
+    token's own outer product, over an fp32 state [dim, dim] per head in a state slot:
+        o_t = (S_(t-1) + diag(u) k_t v_t^T)^T r_t,   S_t = diag(w_t) S_(t-1) + k_t v_t^T
+    w_t = exp(-exp(W_w2 tanh(W_w1 x_w) + w0)) per head and key channel (fp32; the gate's low-rank width is the
+    tensors'). Each of r, k, v, g, w reads its own blend x_s = h + (h' - h) mu_s of the token's input h and the
+    previous token's h' (zeros before the first token; the last token's h is kept in the state slot beside S).
+    Output: every head's o divided by its root mean square, the heads concatenated, times ``norm`` [heads * dim],
+    times silu(W_g x_g), then W_o. spec: heads, dim."""
+    kind = "wkv"
+    cache = "state"
+    SHIFTS = ("r", "k", "v", "g", "w")
+
+    def __init__(self, spec: dict, width: int, eps: float, tensors: dict, device, f32: bool):
+        self.H, self.D = int(spec["heads"]), int(spec["dim"])
+        if self.D > seq.LINEAR_ATTN_MAX_DIM:
+            raise ValueError(f"wkv: the recurrence keeps a state column in registers: dim <= {seq.LINEAR_ATTN_MAX_DIM}")
+        self.eps, self.f32, self.W = eps, f32, width
+        dev = torch.device(device)
+        self.in_rows, self.in_bias = [], {}   # nothing reads the layer's input itself
+        self.mu = torch.stack([tensors["mu." + n].float() for n in self.SHIFTS]).to(dev).contiguous()
+        self.r, self.k, self.v, self.g = (Proj(tensors[n], dev, f32) for n in ("r", "k", "v", "g"))
+        if tensors["w2"].shape[1] != tensors["w1"].shape[0]:
+            raise ValueError("wkv: w1 / w2 disagree on the decay gate's width")
+        self.w1 = Proj(tensors["w1"], dev, f32, allow_packed=False)                      # tanh in its epilogue
+        self.w2 = Proj(tensors["w2"], dev, f32, allow_packed=False, bias=tensors["w0"])  # fp32 logits + w0
+        self.u = _f32(tensors["u"].reshape(self.H, self.D), dev)
+        self.nw = _f32(tensors["norm"], dev)
+        self.o = Proj(tensors["o"], dev, f32)
+
+    @staticmethod
+    def shapes(spec: dict, width: int) -> dict:
+        H, D = spec["heads"], spec["dim"]
+        n = H * D
+        out = {"mu." + s: (width,) for s in ShiftedLinearAttention.SHIFTS}
+        out.update({"r": (n, width), "k": (n, width), "v": (n, width), "g": (n, width), "w1": (None, width), "w2": (n, None),
+                    "w0": (n,), "u": (H, D), "norm": (n,), "o": (width, n)})
+        return out
+
+    def allocate(self, num_blocks: int, block_size: int, num_slots: int, device) -> tuple:
+        """(the recurrence's state, the last token's input) per state slot."""
+        return (torch.zeros(num_slots, self.H, self.D, self.D, dtype=torch.float32, device=device),
+                torch.zeros(num_slots, self.W, dtype=torch.float32, device=device))
+
+    def page_bytes(self, block_size: int) -> int:
+        return 0
+
+    def nbytes(self) -> int:
+        return sum(p.nbytes() for p in (self.r, self.k, self.v, self.g, self.w1, self.w2, self.o))
+
+    def forward(self, h, P, cols, sv, cache) -> torch.Tensor:
+        T = h.shape[0]
+        state, last = cache
+        x = torch.empty(len(self.SHIFTS), T, self.W, dtype=h.dtype, device=h.device)
+        seq.shift_mix(h, last, self.mu, sv.state_slots, sv.context_lens, sv.query_start, x, num_seqs=sv.num_seqs or None)
+        r, k, v, g = self.r(x[0]), self.k(x[1]), self.v(x[2]), self.g(x[3])
+        z = self.w2(self.w1(x[4], act=seq.ACT_TANH), out_f32=True)
+        out = torch.empty(T, self.H * self.D, dtype=h.dtype, device=h.device)
+        seq.linear_attn(r, k, v, g, z, None, 1.0, 1.0, False, self.nw, False, True, state, sv.state_slots, sv.context_lens,
+                        sv.query_start, out, self.eps, num_seqs=sv.num_seqs or None, decay_exp=True, bonus=self.u,
+                        norm_full=True)
+        return self.o(out, out_f32=True)
+
+
 class ParallelMixers:
     """Two mixers side by side on the same input: y = left_scale * left(h) + right_scale * right(h).
     spec: ``left`` / ``right`` = (key of MIXERS, that mixer's spec); tensors under ``left.`` / ``right.``.
@@ -531,20 +664,23 @@ class ParallelMixers:
         return ys[0], self.scales[0], ys[1], self.scales[1]
 
 
-MIXERS = {c.kind: c for c in (LatentAttention, GeneralDelta, WindowAttention, LinearAttention, ParallelMixers)}
+MIXERS = {c.kind: c for c in (LatentAttention, GeneralDelta, WindowAttention, LinearAttention, ShiftedLinearAttention,
+                              ParallelMixers)}
 
 
 # ------------------------------------------------------------------------------------ feed-forwards
 class DenseFF:
-    """down(act(gate h) * (up h)); spec ``act``: "silu" (default) or "gelu_tanh"."""
-    ACTS = {"silu": seq.ACT_SILU_MUL, "gelu_tanh": seq.ACT_GELU_TANH_MUL}
+    """down(act(gate h) * (up h)); spec ``act``: "silu" (default), "gelu_tanh", or "clamped" with ``limit`` L:
+    g = min(gate h, L), u = clamp(up h, -L, L), down(g * sigmoid(ALPHA g) * (u + 1))."""
+    ACTS = {"silu": seq.ACT_SILU_MUL, "gelu_tanh": seq.ACT_GELU_TANH_MUL, "clamped": seq.ACT_CLAMPED_GLU}
+    ALPHA = 1.702
 
     def __init__(self, spec: dict, width: int, tensors: dict, device, f32: bool):
         act = spec.get("act", "silu")
         if act not in self.ACTS:
             raise ValueError(f"dense feed-forward: act {act!r}")
         self.gate_up = Proj(torch.cat([tensors["gate"], tensors["up"]]), device, f32, silu_pair=True,
-                            pair_act=self.ACTS[act])
+                            pair_act=self.ACTS[act], limit=float(spec.get("limit", 0.0)), alpha=self.ALPHA)
         self.down = Proj(tensors["down"], device, f32)
 
     @staticmethod

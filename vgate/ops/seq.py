@@ -215,12 +215,16 @@ def latent_qrope(q, positions, inv_freq, rot_dims: int, qa, H: int, dim: int, ra
     qa.view(T, H, rank + rot)[..., rank:] = _rope_pairs(qr, positions, inv_freq, rot_dims).to(qa.dtype)
 
 
+LATENT_FULL = 1 << 30   # "window" of a latent attention that sees every earlier position
+
+
 def latent_attn(qa, cache, block_tables, context_lens, query_start, ol, scale: float, H: int, rank: int, rot: int,
-                num_seqs: int | None = None, cache_t=None) -> None:
-    """ol[t, h] = sum_j softmax_j(scale * qa[t, h] . cache_j) cache_j[:rank], j <= position(t).
-    With ``cache_t`` (see :func:`latent_write`) bf16 caches run the MFMA kernel."""
+                num_seqs: int | None = None, cache_t=None, window: int = LATENT_FULL, sink=None) -> None:
+    """ol[t, h] = sum_j softmax_j(scale * qa[t, h] . cache_j) cache_j[:rank] over the keys j with
+    0 <= position(t) - j < window. ``sink`` [H] fp32: exp(sink[h]) is added to the softmax denominator (unscaled,
+    once). With ``cache_t`` (see :func:`latent_write`) bf16 caches run the MFMA kernel."""
     if qa.is_cuda:
-        _C().latent_attn(qa, cache, block_tables, context_lens, query_start, ol, scale, H, rank, rot, cache_t)
+        _C().latent_attn(qa, cache, block_tables, context_lens, query_start, ol, scale, H, rank, rot, cache_t, window, sink)
         return
     E = rank + rot
     T = qa.numel() // (H * E)
@@ -238,8 +242,12 @@ def latent_attn(qa, cache, block_tables, context_lens, query_start, ol, scale: f
         rows = flat[(block_tables[s].long()[j // page] * page + j % page)].float()
         sc = torch.einsum("the,je->thj", q3[t0:t1], rows) * scale
         pos = ctx - (t1 - t0) + torch.arange(t1 - t0)
-        sc = sc.masked_fill(j[None, None, :] > pos[:, None, None], float("-inf"))
-        o3[t0:t1] = torch.einsum("thj,jr->thr", torch.softmax(sc, -1), rows[:, :rank]).to(ol.dtype)
+        hidden = (j[None, None, :] > pos[:, None, None]) | (j[None, None, :] <= pos[:, None, None] - window)
+        sc = sc.masked_fill(hidden, float("-inf"))
+        if sink is not None:
+            sc = torch.cat([sc, sink.view(1, H, 1).expand(t1 - t0, H, 1)], -1)
+        p = torch.softmax(sc, -1)[..., :ctx]
+        o3[t0:t1] = torch.einsum("thj,jr->thr", p, rows[:, :rank]).to(ol.dtype)
 
 
 def delta_rule(r, k, v, g, a, wl, w0, ab, nw, state, state_slots, context_lens, query_start, out,
@@ -370,14 +378,80 @@ def hyper_mix(xs: torch.Tensor, y: torch.Tensor | None, mix: torch.Tensor | None
         sum_out.copy_(xs[:, : sum_out.shape[0]].sum(0))
 
 
-def glu_rows(gu: torch.Tensor, out: torch.Tensor, act: int) -> torch.Tensor:
-    """out = act(gu[:, :n]) * gu[:, n:] for a stacked [gate; up] projection (act: ACT_SILU_MUL or ACT_GELU_TANH_MUL)."""
+def glu_rows(gu: torch.Tensor, out: torch.Tensor, act: int, limit: float = 0.0, alpha: float = 1.702) -> torch.Tensor:
+    """out = act(gu[:, :n], gu[:, n:]) for a stacked [gate; up] projection (act: ACT_SILU_MUL, ACT_GELU_TANH_MUL, or
+    ACT_CLAMPED_GLU with ``limit`` and ``alpha``)."""
     if gu.is_cuda:
-        _C().glu_rows(gu, out, act)
+        _C().glu_rows(gu, out, act, limit, alpha)
         return out
     n = out.shape[1]
-    out.copy_(_act(gu[: out.shape[0], :n].float(), gu[: out.shape[0], n:].float(), act, 0.0, 0.0))
+    out.copy_(_act(gu[: out.shape[0], :n].float(), gu[: out.shape[0], n:].float(), act, limit, alpha))
     return out
+
+
+def residual_norm(x: torch.Tensor, y: torch.Tensor, mult: float, w: torch.Tensor | None = None, eps: float = 0.0,
+                  h_out: torch.Tensor | None = None) -> None:
+    """x += mult * y in fp32 (x fp32 [T, W], y fp32 or the activation dtype). With ``w`` [W]: also
+    h_out = x / sqrt(mean(x^2) + eps) * w from the new x, rounded to h_out's dtype."""
+    if x.is_cuda:
+        _C().residual_norm(x, y, mult, w, eps, h_out)
+        return
+    T = y.shape[0]
+    x[:T] += mult * y.float()
+    if w is not None:
+        xf = x[: h_out.shape[0]]
+        h_out.copy_(xf * (1.0 / torch.sqrt(xf.pow(2).mean(-1, keepdim=True) + eps)) * w)
+
+
+def pair_rows(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t] = [a[t], b[t]] (two fp32 [T, W] row sets side by side) rounded to out's dtype."""
+    if a.is_cuda:
+        _C().pair_rows(a, b, out)
+        return out
+    T = out.shape[0]
+    out.copy_(torch.cat([a[:T], b[:T]], -1))
+    return out
+
+
+def shift_mix(h: torch.Tensor, last: torch.Tensor, mu: torch.Tensor, state_slots, context_lens, query_start,
+              out: torch.Tensor, num_seqs: int | None = None) -> None:
+    """Blends of every token's row with the row of the token before it: out[s, t] = h[t] + (h'[t] - h[t]) * mu[s]
+    for the ``mu`` [n, W] fp32 blend vectors, with h' the previous token's h: the row before inside the step, the
+    sequence's ``last`` [slots, W] fp32 row for the first token of a portion, zeros at position 0. Afterwards
+    ``last`` holds the portion's last row. Computed in fp32, rounded once to out's dtype."""
+    if h.is_cuda:
+        _C().shift_mix(h, last, mu, state_slots, context_lens, query_start, out)
+        return
+    S = state_slots.numel() if num_seqs is None else num_seqs
+    for s in range(S):
+        t0, t1 = int(query_start[s]), int(query_start[s + 1])
+        slot = int(state_slots[s])
+        if t1 <= t0 or slot < 0:
+            continue
+        hf = h[t0:t1].float()
+        first = last[slot].clone() if int(context_lens[s]) - (t1 - t0) > 0 else torch.zeros_like(last[slot])
+        prev = torch.cat([first[None], hf[:-1]])
+        out[:, t0:t1] = (hf[None] + (prev - hf)[None] * mu[:, None, :]).to(out.dtype)
+        last[slot] = hf[-1]
+
+
+def map_pair_combine(a: torch.Tensor, lam: float, out_scale: float, eps: float, gate, out: torch.Tensor, H: int, G: int,
+                     V: int) -> None:
+    """Two attention maps per head into one output. ``a`` [T, 2 H V] holds the maps' results grouped (key/value
+    head, map, head in group); per head h: o = a1 - lam * a2, o / sqrt(mean(o^2) + eps) over V, times
+    ``out_scale``, times sigmoid(gate[t, h]) if given; out [T, H V] with the heads in their own order. fp32."""
+    if a.is_cuda:
+        _C().map_pair_combine(a, lam, out_scale, eps, gate, out, H, G, V)
+        return
+    T = out.shape[0]
+    rep = H // G
+    af = a[:T].float().view(T, G, 2, rep, V)
+    o = (af[:, :, 0] - lam * af[:, :, 1]).reshape(T, H, V)
+    o = o * (1.0 / torch.sqrt(o.pow(2).mean(-1, keepdim=True) + eps)) * out_scale
+    o = o.reshape(T, H * V)
+    if gate is not None:
+        o = o * torch.sigmoid(gate[:T].float())
+    out.copy_(o)
 
 
 def post_norm_add(x, y1, w, eps: float, out, s1: float = 1.0, y2=None, s2: float = 1.0, act_out=None, hist=None,
@@ -413,7 +487,7 @@ def _rope_pairs_heads(x: torch.Tensor, pos: torch.Tensor, inv_freq: torch.Tensor
 
 def window_write(q, k, v, qw, kw, eps: float, norm_all: bool, positions, slots, inv_freq, rot_dims: int, v_freq,
                  kc, vc, q_out, H: int, G: int, vt=None, q_head_scale=None, q_temp_coef: float = 0.0,
-                 q_temp_every: int = 1) -> None:
+                 q_temp_every: int = 1, rot_half: bool = False) -> None:
     """Prepare one step's queries, keys and values of a window-attention layer.
     q [T, H * D], k [T, G * D], v [T, G * V] (biases already added). Query / key RMS norm (``qw`` / ``kw``
     None: none; ``norm_all``: over the whole projection with a [heads * D] weight, else per head with a
@@ -422,10 +496,12 @@ def window_write(q, k, v, qw, kw, eps: float, norm_all: bool, positions, slots, 
     query at position p times 1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1). q goes to ``q_out``; keys and values to the paged caches
     kc [pages, G, page, D] / vc [pages, G, page, V] at the tokens' slots (slot < 0: padding row).
     ``vt`` (GPU, bf16): a second copy of the values laid out [pages, G, V, page], the operand layout of
-    the MFMA attention kernel's weighted sum."""
+    the MFMA attention kernel's weighted sum. ``rot_half``: entry i is paired with entry i + rot_dims / 2 instead
+    of 2i with 2i + 1. The value cache may have fewer heads than the key cache (vc.shape[1] divides G: consecutive
+    key heads share a value head); v then is [T, value heads * V]."""
     if q.is_cuda:
         _C().window_write(q, k, v, qw, kw, eps, norm_all, positions, slots, inv_freq, rot_dims, v_freq, kc, vc, q_out, H, G, vt,
-                          q_head_scale, q_temp_coef, q_temp_every)
+                          q_head_scale, q_temp_coef, q_temp_every, rot_half)
         return
     T = q.shape[0]
     D, V, page = kc.shape[3], vc.shape[3], kc.shape[2]
@@ -439,14 +515,16 @@ def window_write(q, k, v, qw, kw, eps: float, norm_all: bool, positions, slots, 
         x = x.view(T, heads, D)
         return x * (1.0 / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps)) * w
 
-    qn = _rope_pairs_heads(norm(qf, qw, H), positions[:T], inv_freq, rot_dims)
+    turn = (lambda x: _rope_halves(x, positions[:T], inv_freq, rot_dims)) if rot_half else \
+        (lambda x: _rope_pairs_heads(x, positions[:T], inv_freq, rot_dims))
+    qn = turn(norm(qf, qw, H))
     if q_head_scale is not None:
         qn = qn * q_head_scale.view(1, H, 1)
     if q_temp_coef != 0.0:
         grow = 1.0 + q_temp_coef * torch.log(torch.floor((positions[:T] + 1).float() / q_temp_every) + 1.0)
         qn = qn * grow.view(T, 1, 1)
-    kn = _rope_pairs_heads(norm(kf, kw, G), positions[:T], inv_freq, rot_dims)
-    vn = vf.view(T, G, V)
+    kn = turn(norm(kf, kw, G))
+    vn = vf.view(T, vc.shape[1], V)
     if v_freq is not None:
         vn = _rope_pairs_heads(vn, positions[:T], v_freq, 2 * v_freq.numel())
     q_out.copy_(qn.reshape(T, H * D))
@@ -482,7 +560,7 @@ def window_pool(kc, vc, kp, vp, positions, block_tables, query_start, pool: int,
 
 def window_attn(q, kc, vc, kp, vp, block_tables, context_lens, query_start, out, scale: float, H: int, window: int,
                 pool: int, sink, v_freq, num_seqs: int | None = None, vt=None, prefill_kernel: int = 0,
-                bias_kind: int = BIAS_NONE, bias_a=None, bias_b=None, gate=None) -> None:
+                bias_kind: int = BIAS_NONE, bias_a=None, bias_b=None, gate=None, softcap: float = 0.0) -> None:
     """out[t, h] = sum_j p_j value_j over the keys position i of token t sees: the tokens j with
     0 <= i - j < window and, with ``pool`` = P > 0, the pooled row of every block b with
     b P + P - 1 <= i - window; p = softmax(scale q . key) over both kinds together, with exp(sink[h]) added
@@ -492,7 +570,9 @@ def window_attn(q, kc, vc, kp, vp, block_tables, context_lens, query_start, out,
     ``BIAS_TABLE``: bias_a[h, min(n, last)] (fp32 [H, distances]). ``gate`` [T, H * V]: the result is
     multiplied by sigmoid(gate). With ``vt`` (see :func:`window_write`) bf16 caches run
     the MFMA kernels (``prefill_kernel``: which one prompt portions take, 0 = tiles staged in LDS for 64 rows,
-    1 = 16 rows per workgroup with the tiles shared out over its waves)."""
+    1 = 16 rows per workgroup with the tiles shared out over its waves). ``softcap`` c > 0: the scaled score s
+    becomes c tanh(s / c) (not together with a distance term). The value caches may have fewer heads than the key
+    cache (consecutive key heads share a value head)."""
     if q.is_cuda:
         parts, scratch = 1, None
         if vt is not None and WINDOW_SPLIT:   # decoded tokens of the MFMA kernel: several workgroups per 16-row tile
@@ -501,7 +581,7 @@ def window_attn(q, kc, vc, kp, vp, block_tables, context_lens, query_start, out,
             if parts > 1:
                 scratch = torch.empty(n, dtype=torch.float32, device=q.device)
         _C().window_attn(q, kc, vc, kp, vp, block_tables, context_lens, query_start, out, scale, H, window, pool, sink, v_freq, vt,
-                         prefill_kernel, bias_kind, bias_a, bias_b, gate, parts, scratch)
+                         prefill_kernel, bias_kind, bias_a, bias_b, gate, parts, scratch, softcap)
         return
     G, page, D, V = kc.shape[1], kc.shape[2], kc.shape[3], vc.shape[3]
     rep = H // G
@@ -516,7 +596,9 @@ def window_attn(q, kc, vc, kp, vp, block_tables, context_lens, query_start, out,
             i = pos0 + t - t0
             lo = max(0, i - window + 1)
             pg, r = _seq_rows(bt, torch.arange(lo, i + 1), page)
-            K, Vv = kc[pg, :, r].float(), vc[pg, :, r].float()           # [n, G, D], [n, G, V]
+            K, Vv = kc[pg, :, r].float(), vc[pg, :, r].float()           # [n, G, D], [n, value heads, V]
+            if Vv.shape[1] != G:
+                Vv = Vv.repeat_interleave(G // Vv.shape[1], dim=1)
             nb = max(0, i - window + 1) // pool if pool else 0
             if nb:
                 e = torch.arange(nb) * pool + pool - 1
@@ -525,6 +607,8 @@ def window_attn(q, kc, vc, kp, vp, block_tables, context_lens, query_start, out,
                 Vv = torch.cat([vp[pg, :, r // pool].float(), Vv])
             qh = q[t].float().view(G, rep, D)
             sc = torch.einsum("grd,ngd->grn", qh, K) * scale               # [G, rep, n]
+            if softcap > 0.0:
+                sc = softcap * torch.tanh(sc / softcap)
             if bias_kind != BIAS_NONE:
                 dist = (i - torch.arange(lo, i + 1))
                 if bias_kind == BIAS_LOG:
@@ -548,7 +632,7 @@ def window_attn(q, kc, vc, kp, vp, block_tables, context_lens, query_start, out,
 def linear_attn(q, k, v, g, z, head_decay, tau: float, q_scale: float, in_silu: bool, nw, norm_all: bool,
                 gate_silu: bool, state, state_slots, context_lens, query_start, out, eps: float,
                 num_seqs: int | None = None, cols_per_lane: int = 0, k_scale: float = 1.0, positions=None, inv_freq=None,
-                rot_dims: int = 0, rot_half: bool = True) -> None:
+                rot_dims: int = 0, rot_half: bool = True, decay_exp: bool = False, bonus=None, norm_full: bool = False) -> None:
     """Decayed outer-product recurrence over state slots, state [slots, H, D, V] fp32:
         S <- diag(a_t) S + k_t v_t^T,  o_t = S^T (q_scale q_t)
     a_t = sigmoid(z_t)^(1 / tau) per key channel (``z`` fp32 [T, H * D]) or the constant head_decay[h];
@@ -557,14 +641,17 @@ def linear_attn(q, k, v, g, z, head_decay, tau: float, q_scale: float, in_silu: 
     multiplied by ``k_scale``. Then RMS norm of o (``nw`` None: no weight) (per head with a [V] weight, or with ``norm_all`` over
     the concatenated heads with a [H * V] weight), times silu(g) or sigmoid(g). A portion that starts at
     position 0 starts from a zero state. ``cols_per_lane`` (GPU): value columns a lane of the scan keeps, 0 =
-    chosen by the launch's size."""
+    chosen by the launch's size. ``decay_exp``: a_t = exp(-exp(z_t)) instead. ``bonus`` [H, D] fp32: the state is read
+    BEFORE its update and the current token's own outer product enters the output through the bonus,
+        o_t = (S_(t-1) + diag(bonus) k_t v_t^T)^T (q_scale q_t),  then  S_t = diag(a_t) S_(t-1) + k_t v_t^T.
+    ``norm_full`` (per-head norm): the weight is [H * V], one entry per output channel."""
     if q.is_cuda:
         H, D, V = state.shape[1], state.shape[2], state.shape[3]
         n = _C().linear_attn_scratch(q.shape[0], state_slots.numel(), H, D, V)
         scratch = torch.empty(n, dtype=torch.float32, device=q.device)
         _C().linear_attn(q, k, v, g, z, head_decay, tau, q_scale, in_silu, nw, norm_all, gate_silu, state, state_slots,
                          context_lens, query_start, out, eps, scratch, cols_per_lane, k_scale, positions, inv_freq,
-                         rot_dims, rot_half)
+                         rot_dims, rot_half, decay_exp, bonus, norm_full)
         return
     H, D, V = state.shape[1], state.shape[2], state.shape[3]
     S = state_slots.numel() if num_seqs is None else num_seqs
@@ -584,16 +671,22 @@ def linear_attn(q, k, v, g, z, head_decay, tau: float, q_scale: float, in_silu: 
             qq, kk = turn(qq, positions[t0:t1], inv_freq, rot_dims), turn(kk, positions[t0:t1], inv_freq, rot_dims)
         qq, kk = qq * q_scale, kk * k_scale
         vv = act(v[t0:t1].float()).view(n, H, V)
-        if z is not None:
+        if z is not None and decay_exp:
+            a = torch.exp(-torch.exp(z[t0:t1].float())).view(n, H, D)
+        elif z is not None:
             a = torch.exp(torch.nn.functional.logsigmoid(z[t0:t1].float()) / tau).view(n, H, D)
         else:
             a = head_decay.view(1, H, 1).expand(n, H, D)
         o = torch.empty(n, H, V)
         for i in range(n):
-            St = a[i][:, :, None] * St + kk[i][:, :, None] * vv[i][:, None, :]
-            o[i] = torch.einsum("hdv,hd->hv", St, qq[i])
+            kv = kk[i][:, :, None] * vv[i][:, None, :]
+            if bonus is not None:
+                o[i] = torch.einsum("hdv,hd->hv", St + bonus[:, :, None] * kv, qq[i])
+            St = a[i][:, :, None] * St + kv
+            if bonus is None:
+                o[i] = torch.einsum("hdv,hd->hv", St, qq[i])
         state[slot] = St
-        one = 1.0 if nw is None else nw
+        one = 1.0 if nw is None else (nw.view(H, V) if norm_full else nw)
         if norm_all:
             of = o.reshape(n, H * V)
             of = of * (1.0 / torch.sqrt(of.pow(2).mean(-1, keepdim=True) + eps)) * one
