@@ -358,7 +358,7 @@ def main():
     ap.add_argument("--design-compare", action="store_true",
                     help="instead of the serving benchmark: prefill / decode tokens/s of a layered hybrid design beside a "
                          "transformer of equal layer sizes (benchmarks/design_compare.py)")
-    ap.add_argument("--design", default="zadirax", choices=["zadirax", "pozalorn", "livitar"], help="the design --design-compare measures")
+    ap.add_argument("--design", default="zadirax", choices=["zadirax", "pozalorn", "livitar", "gefudra"], help="the design --design-compare measures")
     ap.add_argument("--design-beside", default="transformer",
                     help="what --design-compare runs beside the design: transformer (Qwen2 layers of equal sizes) or another design")
     ap.add_argument("--design-only", action="store_true", help="--design-compare without the transformer runs")

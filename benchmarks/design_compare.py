@@ -1,8 +1,8 @@
-"""Prefill and decode throughput of a layered hybrid design (Zadirax, Pozalorn, Livitar) beside the closest
+"""Prefill and decode throughput of a layered hybrid design (Zadirax, Pozalorn, Livitar, Gefudra) beside the closest
 transformer family, or beside another of the designs, at equal layer sizes (random weights, the same number
 of layers), through the engine's own step path.
 
-    python bench.py --design-compare [--design zadirax|pozalorn|livitar] [--design-beside transformer|<design>]
+    python bench.py --design-compare [--design zadirax|pozalorn|livitar|gefudra] [--design-beside transformer|<design>]
                     [--design-sizes 1024,1536] [--design-prefill 2048] [--design-batch 32] [--design-context 512]
 
 Both models run teacher-forced steps (``LLMEngine.replay_step``: cache manager, step metadata, model
@@ -78,7 +78,7 @@ def measure(model: str, overrides: dict | None, prefill: int, batch: int, contex
 _QWEN = {1024: dict(hidden_size=1024, num_heads=8, num_kv_heads=2, intermediate_size=4096, vocab_size=32000, tie_embeddings=False),
          1536: dict(hidden_size=1536, num_heads=12, num_kv_heads=2, intermediate_size=8960, vocab_size=32000, tie_embeddings=False)}
 # design -> (layers of its bench presets, "<design>-bench-<width>")
-DESIGNS = {"zadirax": 4, "pozalorn": 3, "livitar": 3}
+DESIGNS = {"zadirax": 4, "pozalorn": 3, "livitar": 3, "gefudra": 3}
 
 
 def main(sizes: list[int], prefill: int = 2048, batch: int = 32, context: int = 512, design: str = "zadirax",

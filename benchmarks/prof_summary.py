@@ -13,6 +13,7 @@ from collections import defaultdict
 
 
 def short(name: str) -> str:
+    name = name.replace("(anonymous namespace)::", "")
     name = re.sub(r"\(.*$", "", name)  # drop the argument list
     name = name.replace("void ", "").replace("vgate::", "")
     return name[:70]

@@ -428,9 +428,9 @@ def _livitar_preset(name: str, width: int, vocab: int, groups: int, heads: int, 
 
 
 def _gefudra_preset(name: str, width: int, vocab: int, groups: int, heads: int, kv_heads: int, dim: int, ff: int,
-                    kv_rank: int, q_rank: int, window: int, loop_times: int = 2) -> HybridArch:
+                    kv_rank: int, q_rank: int, window: int, loop_times: int = 2, wkv_ff: bool = False) -> HybridArch:
     """Random-init Gefudra models (benchmarks, tests): ``groups`` x [latent attention, two-map attention, wkv
-    (no feed-forward)], the first group's last two layers looped."""
+    (with a feed-forward only if ``wkv_ff``)], the first group's last two layers looped ``loop_times`` times."""
     mlp = {"kind": "dense", "ff": ff, "limit": 7.0}
     lat = {"type": "latent_attention", "mlp": mlp,
            "mixer": {"heads": heads, "dim": dim, "vdim": dim, "kv_rank": kv_rank, "q_rank": q_rank, "scale": dim ** -0.5,
@@ -438,7 +438,7 @@ def _gefudra_preset(name: str, width: int, vocab: int, groups: int, heads: int, 
     att = {"type": "attention", "mlp": mlp,
            "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim // 2, "vdim": dim, "scale": (dim // 2) ** -0.5,
                      "rot": {"base": 10000.0, "dims": dim // 2}, "softcap": 30.0, "diff": 0.5}}
-    wkv = {"type": "wkv", "mlp": None, "mixer": {"heads": heads, "dim": dim}}
+    wkv = {"type": "wkv", "mlp": mlp if wkv_ff else None, "mixer": {"heads": heads, "dim": dim}}
     cfg = {"width": width, "vocab": vocab, "norm": {"eps": 1e-6}, "residual_mult": 0.5, "logit_scale": 1.0,
            "layers": [lat, att, wkv] * groups}
     if loop_times > 0:
@@ -466,10 +466,13 @@ HYBRID_PRESETS = {
     "livitar-bench-1536": lambda: _livitar_preset("livitar-bench-1536", 1536, 32000, 1, 12, 2, 128, 16, 4, 1792, 1792),
     # tests / CPU smoke: odd sizes on purpose
     "gefudra-tiny": lambda: _gefudra_preset("gefudra-tiny", 88, 300, 1, 4, 2, 24, 136, 40, 56, 21),
-    # slices at the layer sizes of real models beside a transformer of equal width (benchmarks/design_compare.py);
-    # no loop, so that three layers run as in the other designs' bench presets
-    "gefudra-bench-1024": lambda: _gefudra_preset("gefudra-bench-1024", 1024, 32000, 1, 8, 2, 128, 4096, 256, 512, 1024, loop_times=0),
-    "gefudra-bench-1536": lambda: _gefudra_preset("gefudra-bench-1536", 1536, 32000, 1, 12, 2, 128, 8960, 512, 768, 1024, loop_times=0),
+    # slices at the layer sizes of real models beside a transformer of equal width (benchmarks/design_compare.py):
+    # three layers with a feed-forward each, as in the other designs' bench presets; the loop runs once (its input
+    # matrix is applied, no layer runs twice)
+    "gefudra-bench-1024": lambda: _gefudra_preset("gefudra-bench-1024", 1024, 32000, 1, 8, 2, 128, 4096, 256, 512, 1024,
+                                                  loop_times=1, wkv_ff=True),
+    "gefudra-bench-1536": lambda: _gefudra_preset("gefudra-bench-1536", 1536, 32000, 1, 12, 2, 128, 8960, 512, 768, 1024,
+                                                  loop_times=1, wkv_ff=True),
     # layer sizes of a ~1.5B model (the width, head size, feed-forward and vocabulary of qwen2.5-1.5b)
     "zadirax-1.5b": lambda: _zadirax_preset("zadirax-1.5b", 1536, 151936, 14, 12, 128, 8960, 32, 4, 2240, 512, 768, 64),
 }
