@@ -23,7 +23,10 @@
 // Waves of a workgroup never meet at a barrier (each loops to its own causal limit), except for a
 // sequence whose rows fit one wave (a decoded token): there the four waves take every fourth key tile
 // of the same rows and merge their partial (max, sum, weighted latent) through LDS, so a lone token's
-// keys are streamed by four waves instead of one.
+// keys are streamed by four waves instead of one. With parts > 1 (steps of decoded tokens: few workgroups), blockIdx.y
+// of up to eight workgroups share such a sequence's key tiles (tile t goes to workgroup (t / 4) mod parts, wave
+// t mod 4); each leaves its merged (max, sum, weighted latent) in an fp32 scratch and latent_attn_merge_kernel
+// rescales and adds them in part order. The number of parts depends on the step's shape alone.
 #include "common.h"
 #include "seq_launchers.h"
 
@@ -258,7 +261,8 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentArgs a, con
                                                                 const int32_t* __restrict__ query_start, int S,
                                                                 const bf16_t* __restrict__ cache_t,
                                                                 bf16_t* __restrict__ ol, int window,
-                                                                const float* __restrict__ sink) {
+                                                                const float* __restrict__ sink, int parts,
+                                                                float* __restrict__ part_o, float* __restrict__ part_ml) {
   __shared__ __attribute__((aligned(16))) bf16_t pl[4][16][40];
   __shared__ float mrg_m[4][16], mrg_l[4][16];
   __shared__ float mrg_o[16][16 * NCT];  // split mode: the merged weighted latent of the 16 rows
@@ -275,6 +279,9 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentArgs a, con
   const int pos0 = context_lens[s] - ntok;
   const int nrows = ntok * H;
   const bool split = nrows <= 16;  // workgroup-uniform: one row tile, keys shared out over the four waves
+  const int part = blockIdx.y;     // (only sequences in split mode are shared out over several workgroups)
+  if (!split && part > 0) return;
+  const int np = split ? parts : 1;
   const int row0 = split ? 0 : tile * 64 + wv * 16;
   if (row0 >= nrows) return;
   const bf16_t* cache = reinterpret_cast<const bf16_t*>(a.cache);
@@ -297,7 +304,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentArgs a, con
     const bool ok = r < nrows;
     limit[i] = ok ? pos0 + r / H + 1 : 0;   // keys [lowest, limit); a row past the last sees none
     lowest[i] = max(0, limit[i] - window);
-    const bool sk = ok && sink != nullptr && (!split || wv == 0);  // the sink counts once
+    const bool sk = ok && sink != nullptr && (!split || (wv == 0 && part == 0));  // the sink counts once
     m[i] = sk ? sink[r % H] * 1.4426950408889634f : -INFINITY;
     lsum[i] = (sk && lr == 0) ? 1.f : 0.f;
   }
@@ -308,7 +315,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentArgs a, con
 #pragma unroll
   for (int ct = 0; ct < NCT; ++ct) O[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int32_t* bt = block_tables + (int64_t)s * max_blocks;
-  for (int j0 = kmin + (split ? 32 * wv : 0); j0 < kmax; j0 += split ? 128 : 32) {
+  for (int j0 = kmin + (split ? 32 * (wv + 4 * part) : 0); j0 < kmax; j0 += split ? 128 * np : 32) {
     int pg0 = bt[j0 >> 4];
     int pg1 = (j0 + 16 < kmax) ? bt[(j0 >> 4) + 1] : pg0;
     pg0 = min(max(pg0, 0), num_pages - 1);
@@ -404,6 +411,19 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentArgs a, con
       }
       __syncthreads();
     }
+    if (np > 1) {  // (workgroup-uniform) hand the partial result on: the merge kernel finishes the rows
+      const int64_t slot = (int64_t)part * gridDim.x + blockIdx.x;
+      float* po = part_o + slot * (16 * 16 * NCT);
+      for (int e = threadIdx.x; e < 16 * 16 * NCT; e += 256) po[e] = (&mrg_o[0][0])[e];
+      if (wv == 0 && lr == 0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          part_ml[(slot * 16 + 4 * lg + i) * 2] = m[i];
+          part_ml[(slot * 16 + 4 * lg + i) * 2 + 1] = lsum[i];
+        }
+      }
+      return;
+    }
     if (wv != 0) return;
 #pragma unroll
     for (int ct = 0; ct < NCT; ++ct)
@@ -426,15 +446,75 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentArgs a, con
   }
 }
 
+// The rows of a split sequence from the partial results of `parts` workgroups: M = max of the parts' maxima (log2
+// units), sums and weighted latents rescaled by 2^(M_p - M) and added in part order, then normalised and stored.
+// vs: the row stride of the parts' weighted latents.
+__global__ __launch_bounds__(256) void latent_attn_merge_kernel(int rank, int H, const int32_t* __restrict__ query_start,
+                                                                 int S, int parts, int vs, const float* __restrict__ part_o,
+                                                                 const float* __restrict__ part_ml,
+                                                                 bf16_t* __restrict__ ol) {
+  int s = -1, base = 0;
+  for (int i = 0; i < S; ++i) {  // the sequence of this workgroup, numbered as in the attention kernel
+    const int nt = ((query_start[i + 1] - query_start[i]) * H + 63) / 64;
+    if ((int)blockIdx.x < base + nt) { s = i; break; }
+    base += nt;
+  }
+  if (s < 0) return;
+  const int t0 = query_start[s], nrows = (query_start[s + 1] - t0) * H;
+  if (nrows > 16) return;  // (not shared out: the attention kernel has stored its rows)
+  constexpr int MAXP = 8;
+  // blockIdx.y: which four rows of the tile
+  for (int e = threadIdx.x; e < 4 * rank; e += blockDim.x) {
+    const int r = 4 * blockIdx.y + e / rank, col = e % rank;
+    if (r >= nrows) continue;
+    float pm[MAXP], plv[MAXP], po[MAXP], M = -INFINITY;
+#pragma unroll
+    for (int p = 0; p < MAXP; ++p) {  // all parts' loads asked for together
+      const int64_t slot = (int64_t)min(p, parts - 1) * gridDim.x + blockIdx.x;
+      pm[p] = p < parts ? part_ml[(slot * 16 + r) * 2] : -INFINITY;
+      plv[p] = part_ml[(slot * 16 + r) * 2 + 1];
+      po[p] = part_o[slot * (16 * vs) + r * vs + col];
+      M = fmaxf(M, pm[p]);
+    }
+    float L = 0.f, y = 0.f;
+#pragma unroll
+    for (int p = 0; p < MAXP; ++p) {
+      const float f = exp2f(pm[p] - M);  // a part that saw no key (or is none): max -inf, factor 0
+      L = fmaf(plv[p], f, L);
+      y = fmaf(po[p], f, y);
+    }
+    ol[((int64_t)(t0 + r / H) * H + r % H) * rank + col] = f2bf(y / L);
+  }
+}
+
 template <int NCT, int NQF>
 void launch_mfma(const LatentArgs& a, const void* qa, int H, float scale, const int32_t* block_tables, int max_blocks,
                  int num_pages, const int32_t* context_lens, const int32_t* query_start, int S, const void* cache_t,
-                 void* ol, int window, const float* sink, hipStream_t st) {
+                 void* ol, int window, const float* sink, int parts, float* scratch, hipStream_t st) {
   const int blocks = (a.T * H + 63) / 64 + S;
-  hipLaunchKernelGGL((latent_attn_mfma_kernel<NCT, NQF>), dim3(blocks), dim3(256), 0, st, a,
+  float* part_o = scratch;
+  float* part_ml = parts > 1 ? scratch + (size_t)parts * blocks * 16 * 16 * NCT : nullptr;
+  hipLaunchKernelGGL((latent_attn_mfma_kernel<NCT, NQF>), dim3(blocks, parts), dim3(256), 0, st, a,
                      reinterpret_cast<const bf16_t*>(qa), H, scale * 1.4426950408889634f, block_tables, max_blocks,
                      num_pages, context_lens, query_start, S, reinterpret_cast<const bf16_t*>(cache_t),
-                     reinterpret_cast<bf16_t*>(ol), window, sink);
+                     reinterpret_cast<bf16_t*>(ol), window, sink, parts, part_o, part_ml);
+  if (parts > 1)
+    hipLaunchKernelGGL(latent_attn_merge_kernel, dim3(blocks, 4), dim3(256), 0, st, a.rank, H, query_start, S, parts, 16 * NCT,
+                       part_o, part_ml, reinterpret_cast<bf16_t*>(ol));
+}
+
+// 16-column tiles / 32-wide query fragments of the instantiation that takes a latent of this size
+void mfma_shape(int rank, int E, int& nct, int& nqf) {
+  if (rank <= 128 && E <= 128) { nct = 8; nqf = 4; }
+  else if (rank <= 128 && E <= 192) { nct = 8; nqf = 6; }
+  else if (rank <= 256 && E <= 256) { nct = 16; nqf = 8; }
+  else if (rank <= 256 && E <= 384) { nct = 16; nqf = 12; }
+  else if (E <= 512) { nct = 32; nqf = 16; }
+  else { nct = 32; nqf = 20; }
+}
+bool mfma_takes(int rank, int rot, int f32, int page) {
+  const int E = rank + rot;
+  return !f32 && page == 16 && rank <= 512 && E <= 640 && E % 8 == 0 && E >= 8;
 }
 
 }  // namespace
@@ -453,15 +533,17 @@ void launch_latent_qrope(const LatentArgs& a, const void* q, int H, int dim, voi
 
 void launch_latent_attn(const LatentArgs& a, const void* qa, int H, float scale, const int32_t* block_tables,
                         int max_blocks, int page, const int32_t* context_lens, const int32_t* query_start, int S,
-                        void* ol, const void* cache_t, int num_pages, int window, const float* sink, hipStream_t st) {
+                        void* ol, const void* cache_t, int num_pages, int window, const float* sink, int parts,
+                        float* scratch, hipStream_t st) {
   if (a.T <= 0 || S <= 0) return;
   const int E = a.rank + a.rot;
-  if (!a.f32 && cache_t != nullptr && page == 16 && a.rank <= 512 && E <= 640 && E % 8 == 0 && E >= 8) {
-#define VG_LAT(NCT, NQF) launch_mfma<NCT, NQF>(a, qa, H, scale, block_tables, max_blocks, num_pages, context_lens, \
-                                               query_start, S, cache_t, ol, window, sink, st)
-    if (a.rank <= 128 && E <= 192) VG_LAT(8, 6);
-    else if (a.rank <= 256 && E <= 384) VG_LAT(16, 12);
-    else VG_LAT(32, 20);
+  if (cache_t != nullptr && mfma_takes(a.rank, a.rot, a.f32, page)) {
+    int nct, nqf;
+    mfma_shape(a.rank, E, nct, nqf);
+    if (parts < 1 || scratch == nullptr) parts = 1;
+#define VG_LAT(NCT, NQF) if (nct == NCT && nqf == NQF) launch_mfma<NCT, NQF>(a, qa, H, scale, block_tables, max_blocks, \
+    num_pages, context_lens, query_start, S, cache_t, ol, window, sink, parts, scratch, st)
+    VG_LAT(8, 4); VG_LAT(8, 6); VG_LAT(16, 8); VG_LAT(16, 12); VG_LAT(32, 16); VG_LAT(32, 20);
 #undef VG_LAT
     return;
   }
@@ -470,6 +552,21 @@ void launch_latent_attn(const LatentArgs& a, const void* qa, int H, float scale,
   const size_t lds = ((size_t)(HC + KT) * (E + 1) + HC * KT + 3 * HC) * sizeof(float);
   hipLaunchKernelGGL(latent_attn_kernel, dim3(a.T, (H + HC - 1) / HC), dim3(256), lds, st, a, qa, H, HC, scale,
                      block_tables, max_blocks, page, context_lens, query_start, S, ol, window, sink);
+}
+
+// Decoded tokens on the MFMA kernel: how many workgroups share a sequence's key tiles (1: no split), chosen from the
+// step's shape so that the launch has about two workgroups per CU, and the scratch floats their partial results take.
+int latent_attn_parts(int T, int S, int H, int rank, int rot, int f32, int page) {
+  if (!mfma_takes(rank, rot, f32, page) || (int64_t)T * H > 16 * (int64_t)S) return 1;
+  const int wg = (T * H + 63) / 64 + S;
+  const int parts = 512 / (wg > 0 ? wg : 1);
+  return parts < 2 ? 1 : (parts > 8 ? 8 : parts);
+}
+size_t latent_attn_part_floats(int T, int S, int H, int rank, int rot, int parts) {
+  if (parts <= 1) return 0;
+  int nct, nqf;
+  mfma_shape(rank, rank + rot, nct, nqf);
+  return (size_t)parts * ((T * H + 63) / 64 + S) * 16 * (16 * nct + 2);
 }
 
 }  // namespace vgate

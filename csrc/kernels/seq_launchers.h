@@ -96,7 +96,12 @@ void launch_latent_qrope(const LatentArgs& a, const void* q, int H, int dim, voi
 // 0 <= position(t) - j < window; sink [H] (null: none): exp(sink[h]) is added to the softmax denominator
 void launch_latent_attn(const LatentArgs& a, const void* qa, int H, float scale, const int32_t* block_tables,
                         int max_blocks, int page, const int32_t* context_lens, const int32_t* query_start, int S,
-                        void* ol, const void* cache_t, int num_pages, int window, const float* sink, hipStream_t st);
+                        void* ol, const void* cache_t, int num_pages, int window, const float* sink, int parts,
+                        float* scratch, hipStream_t st);
+// decoded tokens on the bf16 MFMA kernel: how many workgroups share a sequence's key tiles (1: no split), and the fp32
+// scratch elements launch_latent_attn then needs (parts and scratch must be these for the step's shape)
+int latent_attn_parts(int T, int S, int H, int rank, int rot, int f32, int page);
+size_t latent_attn_part_floats(int T, int S, int H, int rank, int rot, int parts);
 
 struct DeltaArgs {
   const void* r = nullptr; const void* k = nullptr; const void* v = nullptr; const void* g = nullptr;

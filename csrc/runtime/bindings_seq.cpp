@@ -189,7 +189,7 @@ void latent_qrope(const Tensor& q, const Tensor& positions, const Tensor& inv_fr
 
 void latent_attn(const Tensor& qa, const Tensor& cache, const Tensor& block_tables, const Tensor& context_lens,
                  const Tensor& query_start, Tensor& ol, double scale, int64_t H, int64_t rank, int64_t rot,
-                 const OptT& cache_t, int64_t window, const OptT& sink) {
+                 const OptT& cache_t, int64_t window, const OptT& sink, int64_t parts, const OptT& part_scratch) {
   const int f = act_f32(qa, "qa");
   TORCH_CHECK(window >= 1 && window <= (1 << 30), "latent_attn: window 1 .. 2^30");
   const int64_t E = rank + rot;
@@ -212,10 +212,20 @@ void latent_attn(const Tensor& qa, const Tensor& cache, const Tensor& block_tabl
                 cache_t->numel() == cache.size(0) * cache.size(1) * rank, "latent_attn: cache_t bf16 [pages, rank, page]");
     ct = cache_t->data_ptr();
   }
+  float* sp = nullptr;
+  if (parts > 1) {  // only what latent_attn_parts() allows for this launch, with its scratch
+    TORCH_CHECK(ct != nullptr && parts == vgate::latent_attn_parts((int)T, (int)S, (int)H, (int)rank, (int)rot, f, (int)cache.size(1)),
+                "latent_attn: parts must be latent_attn_split()'s for this step");
+    const size_t need = vgate::latent_attn_part_floats((int)T, (int)S, (int)H, (int)rank, (int)rot, (int)parts);
+    TORCH_CHECK(has(part_scratch) && part_scratch->is_cuda() && part_scratch->scalar_type() == torch::kFloat32 &&
+                part_scratch->is_contiguous() && (size_t)part_scratch->numel() >= need, "latent_attn: part_scratch fp32 with ",
+                need, " elements");
+    sp = part_scratch->data_ptr<float>();
+  }
   c10::DeviceGuard guard(qa.device());
   vgate::launch_latent_attn(a, qa.data_ptr(), (int)H, (float)scale, bt, (int)block_tables.size(1), (int)cache.size(1),
                             cl, qs, (int)S, ol.data_ptr(), ct, (int)cache.size(0), (int)window, f32p(sink, "sink", H),
-                            cur_stream());
+                            (int)parts, sp, cur_stream());
 }
 
 void delta_rule(const Tensor& r, const Tensor& k, const Tensor& v, const Tensor& g, const Tensor& a, const Tensor& wl,
@@ -707,7 +717,12 @@ void bind_seq(pybind11::module& m) {
   m.def("latent_attn", &latent_attn, "causal attention over the paged latent cache (absorbed projections)", py::arg("qa"),
         py::arg("cache"), py::arg("block_tables"), py::arg("context_lens"), py::arg("query_start"), py::arg("ol"),
         py::arg("scale"), py::arg("H"), py::arg("rank"), py::arg("rot"), py::arg("cache_t") = py::none(),
-        py::arg("window") = (int64_t)1 << 30, py::arg("sink") = py::none());
+        py::arg("window") = (int64_t)1 << 30, py::arg("sink") = py::none(), py::arg("parts") = 1,
+        py::arg("part_scratch") = py::none());
+  m.def("latent_attn_split", [](int64_t T, int64_t S, int64_t H, int64_t rank, int64_t rot, bool f32, int64_t page) {
+    const int parts = vgate::latent_attn_parts((int)T, (int)S, (int)H, (int)rank, (int)rot, f32 ? 1 : 0, (int)page);
+    return std::make_pair((int64_t)parts, (int64_t)vgate::latent_attn_part_floats((int)T, (int)S, (int)H, (int)rank, (int)rot, parts));
+  }, "workgroups that share a decoded token's key tiles in latent_attn, and the fp32 scratch elements they need");
   m.def("delta_rule", &delta_rule, "generalized delta rule recurrence over state slots + head norm + gate");
   m.def("cast_rows", &cast_rows, "fp32 rows rounded to bf16");
   m.def("glu_rows", &glu_rows, "out = act(gate) * up over a stacked [gate; up] projection", py::arg("gu"), py::arg("out"),

@@ -74,12 +74,12 @@ def config_c():
     """Page-scale geometry on the MFMA kernels' sizes: windows that end inside the third page, exactly at a page
     border and one past it, three passes through the loop, the loop at the end, no loop input before layer 0."""
     return _model(64, 96, [
-        _lat(4, 16, 32, 32, 24, 40, _ff(48)),
-        _att(4, 2, 16, 32, 8, 10000.0, 50.0, 0.6, _ff(48)),
+        _lat(4, 16, 32, 32, 24, 37, _ff(48)),
+        _att(4, 2, 16, 32, 8, 10000.0, 25.0, 0.7, _ff(48)),
         _wkv(2, 16, None),
         _lat(2, 32, 16, 48, 16, 16, _ff(48)),
         _att(2, 2, 32, 16, 32, 500.0, 5.0, 0.2, None),
-        _lat(4, 8, 8, 16, 8, 17, None)], (3, 6, 3), 0.3, 2.0, eps=1e-6)
+        _lat(4, 8, 8, 16, 8, 17, None)], (3, 6, 3), 0.35, 1.5, eps=1e-6)
 
 
 def config_d():
@@ -446,7 +446,7 @@ SCATTERED = [[7, 2, 9, 4, 11, 0, 5, 13, 1, 8, 3, 6, 10, 12, 14, 15, 16, 17, 18, 
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("f32", [True, False])
-@pytest.mark.parametrize("rank,window", [(16, 40), (12, 16), (24, 1), (16, 1 << 30)])
+@pytest.mark.parametrize("rank,window", [(16, 37), (12, 16), (24, 1), (16, 1 << 30)])
 def test_latent_window_and_sink_on_crafted_keys(device, f32, rank, window):
     """The latent attention ops alone: for chosen query positions one cached row is made to dominate (it and the
     query are scaled along a probe direction): the oldest key inside the window, the first one outside it, the

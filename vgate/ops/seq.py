@@ -46,6 +46,7 @@ ACT_NONE, ACT_SILU_MUL, ACT_CLAMPED_GLU, ACT_TANH, ACT_GELU_TANH_MUL = 0, 1, 2, 
 BIAS_NONE, BIAS_LOG, BIAS_TABLE = 0, 1, 2   # distance term of an attention score (see window_attn)
 MAX_STREAMS = 16            # copies of the residual stream hyper_mix takes
 WINDOW_SPLIT = os.environ.get("VGATE_WINDOW_SPLIT", "1") == "1"   # "0": one workgroup per decoded 16-row tile
+LATENT_SPLIT = os.environ.get("VGATE_LATENT_SPLIT", "1") == "1"   # "0": one workgroup per decoded sequence
 LINEAR_ATTN_MAX_DIM = 256   # key channels per head the recurrence kernel keeps in registers (csrc/kernels/linear_attn.hip)
 
 
@@ -224,7 +225,14 @@ def latent_attn(qa, cache, block_tables, context_lens, query_start, ol, scale: f
     0 <= position(t) - j < window. ``sink`` [H] fp32: exp(sink[h]) is added to the softmax denominator (unscaled,
     once). With ``cache_t`` (see :func:`latent_write`) bf16 caches run the MFMA kernel."""
     if qa.is_cuda:
-        _C().latent_attn(qa, cache, block_tables, context_lens, query_start, ol, scale, H, rank, rot, cache_t, window, sink)
+        parts, scratch = 1, None
+        if cache_t is not None and LATENT_SPLIT:   # decoded tokens of the MFMA kernel: several workgroups per sequence
+            T = qa.numel() // (H * (rank + rot))
+            parts, n = _C().latent_attn_split(T, block_tables.shape[0], H, rank, rot, cache.dtype == torch.float32, cache.shape[1])
+            if parts > 1:
+                scratch = torch.empty(n, dtype=torch.float32, device=qa.device)
+        _C().latent_attn(qa, cache, block_tables, context_lens, query_start, ol, scale, H, rank, rot, cache_t, window, sink,
+                         parts, scratch)
         return
     E = rank + rot
     T = qa.numel() // (H * E)
