@@ -479,14 +479,14 @@ def test_latent_window_and_sink_on_crafted_keys(device, f32, rank, window):
         qa[i, n % H] += 5.0 * probe
     kv, qa = kv.to(dt).float(), qa.to(dt).float()
 
-    def want_for(win):
+    def want_for(win, with_sink=True):
         c = oracle.rms(kv.double(), eps, w)
         c = c.to(dt).double() if not f32 else c
         out = torch.zeros(T, H, rank, dtype=torch.float64)
         for i in range(T):
             lo = max(0, i - win + 1)
             for h in range(H):
-                p = oracle.sink_softmax((c[lo:i + 1] @ qa[i, h].double()) * scale, float(sink[h]))
+                p = oracle.sink_softmax((c[lo:i + 1] @ qa[i, h].double()) * scale, float(sink[h]) if with_sink else None)
                 out[i, h] = p @ c[lo:i + 1]
         return out.float()
 
@@ -508,6 +508,7 @@ def test_latent_window_and_sink_on_crafted_keys(device, f32, rank, window):
                 done += n
             assert rel(torch.cat(outs), want) < (3e-5 if f32 else 2e-2), (len(steps), mfma)
     # the crafted keys matter: a window one token longer or shorter, or no sink, moves the answer
+    assert rel(want_for(window, with_sink=False), want) > 0.02
     if not full:
         assert rel(want_for(window + 1), want) > 0.02
     if window > 1 and not full:
